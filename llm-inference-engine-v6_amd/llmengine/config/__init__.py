@@ -2,11 +2,12 @@ from .base import ConfigError, KeyReader, read_model_json
 from .llama import LlamaConfig, RopeScaling
 from .rilonex import RilonexConfig
 from .bidirax import BidiraxConfig
+from .zetonex import ZetonexConfig
 from .registry import (Architecture, architecture_name, known_architectures, load_config,
                        parse_config, register_architecture, resolve)
 
 __all__ = [
-    "ConfigError", "KeyReader", "read_model_json", "LlamaConfig", "RopeScaling", "RilonexConfig", "BidiraxConfig", "Architecture",
+    "ConfigError", "KeyReader", "read_model_json", "LlamaConfig", "RopeScaling", "RilonexConfig", "BidiraxConfig", "ZetonexConfig", "Architecture",
     "architecture_name", "known_architectures", "load_config", "parse_config",
     "register_architecture", "resolve",
 ]

@@ -22,6 +22,7 @@ class LayerCall:
     layer: int
     cache: int | None = None        # cache id; None: the layer's own (its index)
     write_cache: bool = True
+    enter: bool = False             # the model's pass-input map runs in front of this call (the first layer of a pass)
 
     @property
     def cache_id(self) -> int:
@@ -32,18 +33,24 @@ class DecoderModel(Part):
     graph_safe = True
 
     def __init__(self, config, embedding: TokenEmbedding, layers: list[Block], final_norm: Norm,
-                 head: Head, schedule: list[LayerCall] | None = None, names: dict | None = None, streams: int = 0):
+                 head: Head, schedule: list[LayerCall] | None = None, names: dict | None = None, streams: int = 0,
+                 pass_input: Part | None = None):
         self.config = config
         # streams > 0: the residual is kept as that many streams [streams, T, H] (blocks that know how read and
         # write them); every stream starts as the embedding, and the final norm reads their sum
         self.streams = int(streams)
         self.embedding, self.layers, self.final_norm, self.head = embedding, list(layers), final_norm, head
         self.schedule = list(schedule) if schedule is not None else [LayerCall(i) for i in range(len(layers))]
+        # what runs in front of the calls marked `enter`: forward(h, h0, step) replaces the stream h, given the
+        # embedding's output h0 (a stack of layers that runs several passes over the same weights)
+        self.pass_input = pass_input
+        if any(call.enter for call in self.schedule) and (pass_input is None or self.streams):
+            raise ValueError("a schedule with passes needs the model's pass-input map (and a single stream)")
         for call in self.schedule:
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"schedule names layer {call.layer}, the model has {len(self.layers)}")
         self.names = {"embedding": "model.embed_tokens", "layers": "model.layers", "final_norm": "model.norm",
-                      "head": "lm_head"}
+                      "head": "lm_head", "pass_input": "pass_input"}
         if names:
             self.names.update(names)
 
@@ -56,6 +63,8 @@ class DecoderModel(Part):
             out[n["layers"].format(i) if "{}" in n["layers"] else f"{n['layers']}.{i}"] = layer
         out[n["final_norm"]] = self.final_norm
         out[n["head"]] = self.head
+        if self.pass_input is not None:
+            out[n["pass_input"]] = self.pass_input
         return out
 
     def aliases(self):
@@ -117,8 +126,15 @@ class DecoderModel(Part):
         else:
             h = step.buffer("model.hidden", (T, self.hidden_size), torch.float32)
             self.embedding.forward(step.tokens, h, step)
+        h0 = None
+        if self.pass_input is not None and any(call.enter for call in self.schedule):
+            # the embedding's output is read again in front of every pass
+            h0 = step.buffer("model.embedded", (T, self.hidden_size), torch.float32)
+            self.embedding.forward(step.tokens, h0, step)
         for i, call in enumerate(self.schedule):
             layer = self.layers[call.layer]
+            if call.enter:
+                self.pass_input.forward(h, h0, step)
             if hasattr(layer, "next_block"):
                 # (a block that can hand the streams' next read on is told which layer runs behind it in this pass)
                 layer.next_block = self.layers[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None

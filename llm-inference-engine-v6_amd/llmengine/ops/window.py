@@ -1,0 +1,174 @@
+"""Python faces of the kernels for softmax attention with windows that keep the first tokens, several score maps
+per value head, capped scores and key and value sizes that differ (csrc/window_attention*.hip), and of the small
+kernels around feed-forward layers with biases, clamped gates and experts chosen by a table (csrc/feed_forward.hip).
+As everywhere in ops: operands are checked on the host, then the kernel is launched on the current stream."""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .lib import KernelError, check, code, declare, entry, ptr, require, stream
+
+_vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+_FLOATS = (torch.float32, torch.bfloat16)
+WINDOW_ATTENTION_MAX_ENTRIES = 256          # entries of a key or value head that the kernels hold
+FINISH_MODES = {"plain": 0, "gate": 1, "difference": 2}
+BIAS_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2, "swish_clamped": 3}
+
+declare("llme_qk_prepare", [_vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _f, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i,
+                            _i, _i, _vp])
+declare("llme_window_attention", [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i, _vp])
+declare("llme_window_attention_finish", [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _f, _f, _f, _vp, _i, _i, _vp])
+declare("llme_gated_bias_act", [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _f, _vp])
+declare("llme_add_row_bias", [_vp, _vp, _i, _i, _i, _vp])
+declare("llme_table_route", [_vp, _vp, _vp, _vp, _i, _i, _vp])
+declare("llme_concat_rows", [_vp, _vp, _vp, _i, _i, _i, _vp])
+
+
+def _columns(p: torch.Tensor, name: str) -> int:
+    """A 32-bit matrix whose rows may be wider than what is read of them: returns the row stride."""
+    if not isinstance(p, torch.Tensor) or not p.is_cuda or p.dtype != torch.float32 or p.dim() != 2 or p.stride(1) != 1:
+        raise KernelError(f"{name}: a 32-bit matrix on the GPU with unit column stride")
+    return p.stride(0)
+
+
+def qk_prepare(p: torch.Tensor, step, block_table: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+               nq: int, k_col: int, v_col: int | None, inv_freq: torch.Tensor | None, rot: int, wq: torch.Tensor | None = None,
+               wk: torch.Tensor | None = None, eps: float = 0.0) -> None:
+    """Rows p [T, ..] (32-bit: nq query heads of dk entries at column 0, the key heads at k_col, the value heads at
+    v_col; v_col None: a value head is the key head as projected) -> q_out [T, nq dk] and the cache entries of the
+    rows' tokens: k_cache [pages, nk, page, dk], v_cache [pages, nv, dv, page]. wq, wk [dk]: every query and key
+    head is divided by its root mean square (eps inside the root) and multiplied by the weight first. Then entry
+    i < rot / 2 of a query or key head turns with entry i + rot / 2 by position * inv_freq[i]."""
+    T = p.shape[0]
+    ld = _columns(p, "p")
+    require(k_cache, "k_cache", _FLOATS, (None, None, None, None))
+    _, nk, page, dk = k_cache.shape
+    require(v_cache, "v_cache", k_cache.dtype, (k_cache.shape[0], None, None, page))
+    nv, dv = v_cache.shape[1], v_cache.shape[2]
+    require(q_out, "q_out", k_cache.dtype, (T, nq * dk))
+    require(block_table, "block_table", torch.int32, (None, None))
+    need = max(nq * dk, k_col + nk * dk, (v_col + nv * dv) if v_col is not None else 0)
+    if p.shape[1] < need:
+        raise KernelError(f"qk_prepare: rows of {p.shape[1]} columns hold no {need}")
+    if v_col is None and (nk != nv or dk != dv):
+        raise KernelError("qk_prepare: values that are the keys need as many value heads of the same size")
+    if rot:
+        require(inv_freq, "inv_freq", torch.float32, (rot // 2,))
+    if (wq is None) != (wk is None):
+        raise KernelError("qk_prepare: query and key norm come together")
+    if wq is not None:
+        require(wq, "wq", _FLOATS, (dk,))
+        require(wk, "wk", wq.dtype, (dk,))
+    check(entry("llme_qk_prepare")(ptr(p), ld, nq, nk, nv, dk, dv, int(k_col), -1 if v_col is None else int(v_col), ptr(wq), ptr(wk),
+                                   code(wq.dtype) if wq is not None else 0, float(eps), ptr(inv_freq) if rot else None, int(rot),
+                                   ptr(step.positions), ptr(step.seq_idx), ptr(block_table), block_table.shape[1], ptr(q_out),
+                                   code(q_out.dtype), ptr(k_cache), ptr(v_cache), code(k_cache.dtype), page, T, stream()),
+          "qk_prepare")
+
+
+_fast_window_attention = None       # set by ops/window_mfma.py: returns the number of runs, or 0 if it declines
+
+
+def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, step, block_table: torch.Tensor, nq: int,
+                     scale: float, softcap: float = 0.0, window: int = 0, keep_first: int = 0):
+    """Every (token, query head) of the step over the keys of its request that it may see. Returns (part_o
+    [runs, T, nq, dv], part_ml [runs, T, nq, 2]): per run of keys the unscaled weighted values, the maximum and the
+    sum, which `window_attention_finish` joins."""
+    T = q.shape[0]
+    require(k_cache, "k_cache", _FLOATS, (None, None, None, None))
+    _, nk, page, dk = k_cache.shape
+    require(v_cache, "v_cache", k_cache.dtype, (k_cache.shape[0], None, None, page))
+    nv, dv = v_cache.shape[1], v_cache.shape[2]
+    require(q, "q", k_cache.dtype, (T, nq * dk))
+    require(block_table, "block_table", torch.int32, (None, None))
+    if nk % nv or nq % nk:
+        raise KernelError(f"window attention: {nq} query, {nk} key and {nv} value heads do not divide")
+    if max(dk, dv) > WINDOW_ATTENTION_MAX_ENTRIES:
+        raise KernelError(f"window attention: heads of {dk} and {dv} entries are beyond the kernels' {WINDOW_ATTENTION_MAX_ENTRIES}")
+    if _fast_window_attention is not None:
+        parts = _fast_window_attention(q, k_cache, v_cache, step, block_table, nq, scale, softcap, window, keep_first)
+        if parts is not None:
+            return parts
+    part_o = step.buffer("window_attention.part_o", (1, T, nq, dv), torch.float32)
+    part_ml = step.buffer("window_attention.part_ml", (1, T, nq, 2), torch.float32)
+    check(entry("llme_window_attention")(ptr(q), code(q.dtype), ptr(k_cache), ptr(v_cache), code(k_cache.dtype), ptr(part_o),
+                                         ptr(part_ml), ptr(step.positions), ptr(step.seq_idx), ptr(block_table),
+                                         block_table.shape[1], T, nq, nk, nv, dk, dv, page, float(scale), float(softcap),
+                                         int(window), int(keep_first), stream()), "window_attention")
+    return part_o, part_ml
+
+
+def window_attention_finish(part_o: torch.Tensor, part_ml: torch.Tensor, out: torch.Tensor, heads: int, mode: str = "plain",
+                            gate: torch.Tensor | None = None, lam: float = 0.0, eps: float = 0.0, out_scale: float = 1.0) -> None:
+    """out [T, heads dv] (a view with its own row stride may be given) from the runs' parts. mode "gate": times
+    sigmoid(gate), gate [T, heads dv] 32-bit (also a view); "difference": a head's two maps as a_1 - lam a_2, divided
+    by the root mean square over the head's entries (eps inside the root), times out_scale."""
+    require(part_o, "part_o", torch.float32, (None, None, None, None))
+    runs, T, nq, dv = part_o.shape
+    require(part_ml, "part_ml", torch.float32, (runs, T, nq, 2))
+    maps = 2 if mode == "difference" else 1
+    if mode not in FINISH_MODES or nq != heads * maps:
+        raise KernelError(f"window_attention_finish: mode {mode!r} with {nq} query heads for {heads} heads")
+    if (not isinstance(out, torch.Tensor) or not out.is_cuda or out.dtype not in _FLOATS or out.dim() != 2 or out.stride(1) != 1
+            or tuple(out.shape) != (T, heads * dv)):
+        raise KernelError(f"window_attention_finish: out must be [T, {heads * dv}] with unit column stride")
+    ld_gate = 0
+    if mode == "gate":
+        ld_gate = _columns(gate, "gate")
+        if tuple(gate.shape) != (T, heads * dv):
+            raise KernelError(f"window_attention_finish: gate must be [T, {heads * dv}]")
+    check(entry("llme_window_attention_finish")(ptr(part_o), ptr(part_ml), runs, T, heads, maps, dv, FINISH_MODES[mode],
+                                                ptr(gate) if mode == "gate" else None, ld_gate, float(lam), float(eps),
+                                                float(out_scale), ptr(out), code(out.dtype), out.stride(0), stream()),
+          "window_attention_finish")
+
+
+# --- feed-forward layers with biases, clamped gates, experts by table --------------------------------
+def gated_bias_act(gu: torch.Tensor, out: torch.Tensor, group: int, activation: str, bias: torch.Tensor | None = None,
+                   limit: float = 0.0, alpha: float = 1.0) -> None:
+    """out [T, FF] = act(gate + b) * (up + b) from gu [T, 2 FF] 32-bit with gate and up columns in alternating groups
+    of `group` (bias [2 FF] in the same order). "swish_clamped": g = min(gate, limit), u = clamp(up, -limit, limit),
+    out = g sigmoid(alpha g) (u + 1)."""
+    require(out, "out", _FLOATS, (None, None))
+    T, FF = out.shape
+    ld = _columns(gu, "gu")
+    if gu.shape[0] != T or gu.shape[1] < 2 * FF:
+        raise KernelError(f"gated_bias_act: gu {tuple(gu.shape)} does not hold [T, {2 * FF}]")
+    if activation not in BIAS_ACTIVATIONS:
+        raise KernelError(f"gated_bias_act: {activation!r} is none of {sorted(BIAS_ACTIVATIONS)}")
+    if group <= 0 or FF % group:
+        raise KernelError(f"gated_bias_act: group {group} does not divide the width {FF}")
+    if bias is not None:
+        require(bias, "bias", _FLOATS, (2 * FF,))
+    check(entry("llme_gated_bias_act")(ptr(gu), ld, ptr(bias), code(bias.dtype) if bias is not None else 0, ptr(out), code(out.dtype),
+                                       T, FF, group, BIAS_ACTIVATIONS[activation], float(limit), float(alpha), stream()),
+          "gated_bias_act")
+
+
+def add_row_bias(x: torch.Tensor, bias: torch.Tensor) -> None:
+    """x[t, :] += bias for every row of the 32-bit matrix x."""
+    require(x, "x", torch.float32, (None, None))
+    require(bias, "bias", _FLOATS, (x.shape[1],))
+    check(entry("llme_add_row_bias")(ptr(x), ptr(bias), code(bias.dtype), x.shape[0], x.shape[1], stream()), "add_row_bias")
+
+
+def table_route(table: torch.Tensor, tokens: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor) -> None:
+    """ids[t] = table[tokens[t]] (the experts of a token's id), wts = 1 / top."""
+    require(table, "table", torch.int32, (None, None))
+    top = table.shape[1]
+    T = tokens.shape[0]
+    require(tokens, "tokens", torch.int32, (T,))
+    require(ids, "ids", torch.int32, (T, top))
+    require(wts, "wts", torch.float32, (T, top))
+    check(entry("llme_table_route")(ptr(table), ptr(tokens), ptr(ids), ptr(wts), T, top, stream()), "table_route")
+
+
+def concat_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> None:
+    """out [T, 2 H] = [a | b] for 32-bit a, b [T, H], in out's type."""
+    require(a, "a", torch.float32, (None, None))
+    T, H = a.shape
+    require(b, "b", torch.float32, (T, H))
+    require(out, "out", _FLOATS, (T, 2 * H))
+    check(entry("llme_concat_rows")(ptr(a), ptr(b), ptr(out), code(out.dtype), T, H, stream()), "concat_rows")

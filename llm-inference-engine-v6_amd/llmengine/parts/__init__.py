@@ -6,7 +6,7 @@ from .rope import RotaryEmbedding, inverse_frequencies
 from .embedding import Embedding, OutputHead
 from .mlp import GatedMLP
 from .attention import Attention
-from .block import PreNormBlock, SandwichBlock
+from .block import ParallelBlock, PreNormBlock, SandwichBlock
 from .projected import ParallelMixer, ProjectedMixer
 from .rglru import RGLRU
 from .delta import GatedDeltaRule
@@ -14,10 +14,12 @@ from .sigmoid_attention import SigmoidAttention
 from .hyper import HyperConnectionBlock
 from .latent_attention import LatentAttention
 from .moe import MixtureOfExperts
+from .window_attention import WindowAttention
+from .reentry import PassInput
 
 __all__ = ["PAGE", "Block", "CacheSpec", "FeedForward", "LayerCache", "Mixer", "Norm", "ParamSpec", "Part",
            "Placement", "PositionEncoding", "TokenEmbedding", "Head", "LayerSpec", "PartChoice", "build_layer", "make_part",
            "register_part", "registered", "RMSNorm", "RotaryEmbedding", "inverse_frequencies", "Embedding",
            "OutputHead", "GatedMLP", "Attention", "PreNormBlock", "ParallelMixer", "ProjectedMixer", "RGLRU", "GatedDeltaRule",
            "SigmoidAttention", "HyperConnectionBlock", "CenteredRMSNorm", "SandwichBlock", "LatentAttention",
-           "MixtureOfExperts"]
+           "MixtureOfExperts", "WindowAttention", "PassInput", "ParallelBlock"]

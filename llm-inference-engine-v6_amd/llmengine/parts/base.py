@@ -36,7 +36,8 @@ import torch
 class ParamSpec:
     """A tensor a part reads from the checkpoint: its exact shape there, and how a
     random model fills it ("linear": N(0, std); "norm": N(mean, std) around one; "identity": the
-    unit matrix plus N(0, std); "taps": N(0, 1/2), for the few taps of a short convolution). A
+    unit matrix plus N(0, std); "taps": N(0, 1/2), for the few taps of a short convolution; "table:<n>": an integer
+    table whose rows hold distinct numbers below n). A
     dimension that only the checkpoint knows (a rank no configuration names) is None: any size
     fits, and the part reads it off the tensor when it loads."""
     shape: tuple[int | None, ...]

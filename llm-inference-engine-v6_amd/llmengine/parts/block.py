@@ -109,5 +109,36 @@ class SandwichBlock(Block):
             step.extra["block.normed is for"] = id(self.next_block)
 
 
+class ParallelBlock(Block):
+    """One norm whose output both sublayers read: h += mixer(norm(h)) + ffn(norm(h)). Both sublayers add into the
+    32-bit stream (their last products accumulate), the mixer first."""
+    graph_safe = True
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward | None, mixer_norm: Norm, ffn_norm: Norm | None = None,
+                 names: dict | None = None):
+        if ffn_norm is not None:
+            raise ValueError("a parallel block has one norm: its feed-forward reads the mixer's")
+        self.mixer, self.feed_forward, self.mixer_norm = mixer, feed_forward, mixer_norm
+        self.names = {"mixer_norm": "norm1", "mixer": "mix", "feed_forward": "mlp"}
+        if names:
+            self.names.update(names)
+
+    def children(self):
+        n = self.names
+        out = {n["mixer_norm"]: self.mixer_norm, n["mixer"]: self.mixer}
+        if self.feed_forward is not None:
+            out[n["feed_forward"]] = self.feed_forward
+        return out
+
+    def forward(self, h, step, cache, write_cache=True):
+        T, H = h.shape
+        x = step.buffer("block.normed", (T, H), step.act_dtype)
+        self.mixer_norm.forward(h, x)
+        self.mixer.forward(x, step, cache, h, True, write_cache)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(x, step, h, True)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)
 register_part("block", "sandwich", SandwichBlock)

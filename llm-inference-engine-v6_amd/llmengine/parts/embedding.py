@@ -38,8 +38,10 @@ class Embedding(TokenEmbedding):
 class OutputHead(Head):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding | None = None, tensor: str = "weight"):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding | None = None, tensor: str = "weight",
+                 scale: float = 1.0):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.scale = float(scale)       # a multiplier on the logits, applied in 32-bit
         self.tied_to = tied_to
         self.tensor = tensor
         self._weight: torch.Tensor | None = None
@@ -64,11 +66,15 @@ class OutputHead(Head):
 
     def forward(self, x: torch.Tensor, out: torch.Tensor, step=None) -> None:
         ops.gemm(x, self.weight, out, choices=getattr(step, "choices", None))
+        if self.scale != 1.0:
+            ops.scale_(out, self.scale)
 
     def forward_normed_rows(self, h: torch.Tensor, rows: torch.Tensor, norm, out: torch.Tensor, step=None) -> None:
         """Logits of the chosen rows of the 32-bit stream, the final norm applied inside the product."""
         weight, eps = norm.fused_rms()
         ops.gemv_norm(h, weight, eps, self.weight, out, rows=rows)
+        if self.scale != 1.0:
+            ops.scale_(out, self.scale)
 
 
 register_part("embedding", "table", Embedding)

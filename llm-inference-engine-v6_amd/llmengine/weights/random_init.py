@@ -33,6 +33,10 @@ def random_tensor(name: str, shape: tuple[int, ...], init: str, seed: int, dtype
                          "name it in the configuration")
     gen = torch.Generator(device="cpu")
     gen.manual_seed(_tensor_seed(seed, name))
+    if init.startswith("table:"):
+        # rows of distinct integers below the number behind the colon (a token id's experts)
+        n = int(init.split(":")[1])
+        return torch.stack([torch.randperm(n, generator=gen)[:shape[1]] for _ in range(shape[0])]).to(torch.int32)
     if init == "identity":
         t = torch.randn(shape, generator=gen, dtype=torch.float32) * std + torch.eye(shape[-2], shape[-1])
     elif init == "taps":
@@ -71,6 +75,7 @@ def write_random_model(config_dict: dict, out_dir: str, seed: int, dtype: torch.
         return random_tensor(name, s.shape, s.init, seed, dtype, std, norm_mean, norm_std)
 
     write_safetensors(os.path.join(out_dir, "model.safetensors"),
-                      {n: (dtype, tuple(s.shape)) for n, s in specs.items()}, produce,
+                      {n: (torch.int32 if s.init.startswith("table:") else dtype, tuple(s.shape)) for n, s in specs.items()},
+                      produce,
                       metadata={"format": "pt", "seed": str(seed)})
     return out_dir
