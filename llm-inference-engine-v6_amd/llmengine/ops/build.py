@@ -34,6 +34,7 @@ SOURCE_FLAGS = {
     "attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "latent_attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "window_attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 

@@ -68,7 +68,54 @@ def qk_prepare(p: torch.Tensor, step, block_table: torch.Tensor, q_out: torch.Te
           "qk_prepare")
 
 
-_fast_window_attention = None       # set by ops/window_mfma.py: returns the number of runs, or 0 if it declines
+declare("llme_window_attention_mfma", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
+                                       _i, _vp])
+WINDOW_MFMA_MAX_ENTRIES = 128       # entries of a key or value head that the matrix-core kernel holds
+WINDOW_MFMA_MAX_RUNS = 32
+
+
+def window_mfma_fits(k_cache: torch.Tensor, v_cache: torch.Tensor, choices=None) -> bool:
+    """Whether the matrix-core kernel takes this cache: bfloat16, key entries a multiple of 8 and value entries a multiple
+    of 16, both up to 128, pages a multiple of 16 tokens."""
+    from .choices import DEFAULT
+    dk, dv, page = k_cache.shape[3], v_cache.shape[2], k_cache.shape[2]
+    return ((choices or DEFAULT).fast_attention and k_cache.dtype == torch.bfloat16 and dk % 8 == 0 and dv % 16 == 0
+            and max(dk, dv) <= WINDOW_MFMA_MAX_ENTRIES and page % 16 == 0)
+
+
+def window_runs(step, rows_per_token: int, key_heads: int, window: int, keep_first: int) -> tuple[int, int]:
+    """(the most tokens a request brings, runs to cut a tile's keys into) for the matrix-core kernel: enough wavefronts
+    for four a compute unit, a run no shorter than a block of 32 keys. A step of single tokens plans for requests of
+    up to step.plan_len keys where that is set (the step may be recorded and replayed for longer requests)."""
+    from . import mfma
+    decode = step.num_tokens == step.num_seqs
+    max_new = 1 if decode else max(step.new_lens)
+    if decode and step.plan_len is not None:
+        keys = step.plan_len
+    else:
+        keys = max(c + n for c, n in zip(step.ctx_lens, step.new_lens))
+    if window:
+        keys = min(keys, window + (16 + rows_per_token - 1) // rows_per_token + min(keep_first, keys))
+    tiles = sum((n * rows_per_token + 15) // 16 for n in step.new_lens) * key_heads
+    blocks = (keys + 31) // 32 + 1
+    return max_new, max(1, min(WINDOW_MFMA_MAX_RUNS, (4 * mfma.compute_units()) // max(tiles, 1), blocks))
+
+
+def _fast_window_attention(q, k_cache, v_cache, step, block_table, nq, scale, softcap, window, keep_first):
+    from .choices import choices_of
+    if not window_mfma_fits(k_cache, v_cache, choices_of(step)):
+        return None
+    T = q.shape[0]
+    _, nk, page, dk = k_cache.shape
+    nv, dv = v_cache.shape[1], v_cache.shape[2]
+    max_new, runs = window_runs(step, nq // nk, nk, window, keep_first)
+    part_o = step.buffer("window_attention.part_o", (runs, T, nq, dv), torch.float32)
+    part_ml = step.buffer("window_attention.part_ml", (runs, T, nq, 2), torch.float32)
+    check(entry("llme_window_attention_mfma")(ptr(q), ptr(k_cache), ptr(v_cache), ptr(part_o), ptr(part_ml), ptr(step.positions),
+                                              ptr(step.q_start), ptr(block_table), block_table.shape[1], T, step.num_seqs, max_new,
+                                              nq, nk, nv, dk, dv, page, float(scale), float(softcap), int(window), int(keep_first),
+                                              runs, stream()), "window_attention_mfma")
+    return part_o, part_ml
 
 
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, step, block_table: torch.Tensor, nq: int,
