@@ -18,7 +18,9 @@ measurements at further sizes and context lengths; the default run is the 1B sha
 
 `--phase design` runs the Rilonex design (recurrent, delta-rule and softmax-free attention layers around
 a residual in several streams) beside Llama with layers of the same sizes: prefill and decode of both;
-`--design bidirax` the Bidirax design instead (latent attention, rotated and windowed, dense and expert feed-forwards).
+`--design bidirax` the Bidirax design instead (latent attention, rotated and windowed, dense and expert feed-forwards),
+`--design zetonex` the Zetonex design (windowed attention with two score maps or with keys as values, dense feed-forwards
+with biases and clamped experts chosen by a table, a stretch of layers that runs two passes).
 
 `--phase mixed` times one step of continuous batching (a prompt portion beside decoded tokens of
 other requests), `--phase portion` portions of one long prompt. `--phase serve` is another workload (with `--shape 3b`: 32 requests with prompts of 64 to 3,072
@@ -116,6 +118,29 @@ def bidirax_at(width: int, ff: int, heads: int, layers: int, vocab: int, only: s
             "layers": out}
 
 
+def zetonex_at(width: int, ff: int, heads: int, layers: int, vocab: int, only: str = "") -> dict:
+    """Zetonex layers of a Llama layer's width, heads and active feed-forward size: differential attention (half the heads,
+    two score maps of 64 each over values of 128, capped scores, a window of 1,024) with a dense feed-forward with biases,
+    then attention whose values are its keys (a window of 1,024 that keeps the first 4 tokens, an output gate) with 16
+    clamped experts chosen by a table (2 a token, half the feed-forward size each). Without `only` the first two layers
+    run two passes, so that `layers` layer runs come from layers - 2 layers."""
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": ff // 2, "limit": 7.0}}
+    diff = {"heads": max(1, heads // 2), "kv_heads": max(1, heads // 8), "dim": 64, "vdim": 128, "scale": 0.125, "diff": 0.3,
+            "softcap": 50.0, "mask": {"size": 1024},
+            "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    gated = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125,
+             "mask": {"size": 1024, "keep_first": 4}, "rot": {"base": 10000.0, "dims": 32}}
+    kinds = {"differential": {"type": "attention_2", "mixer": diff, "mlp": dense}, "gated": {"type": "attention", "mixer": gated, "mlp": moe}}
+    out = {"architecture": "Zetonex", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_scale": 1.0}
+    if only or layers < 4:
+        out["layers"] = [kinds[only or ("differential", "gated")[i % 2]] for i in range(layers)]
+    else:
+        out["layers"] = [kinds[("differential", "gated")[i % 2]] for i in range(layers - 2)]
+        out["loop"] = {"start": 0, "stop": 2, "times": 2}
+    return out
+
+
 def design(args) -> int:
     """Prefill (one prompt of --prefill-tokens) and decode (--batch requests at --context) of the Rilonex design and of
     Llama with layers of the same width, feed-forward size and number of heads: tokens/s of both and their ratio, per
@@ -129,6 +154,7 @@ def design(args) -> int:
         width, ff, heads = DESIGN_SIZES[size]
         row = {"size": size, "width": width, "ff": ff, "heads": heads, "layers": layers}
         other = (bidirax_at(width, ff, heads, layers, vocab, only=args.design_only) if args.design == "bidirax"
+                 else zetonex_at(width, ff, heads, layers, vocab, only=args.design_only) if args.design == "zetonex"
                  else rilonex_at(width, ff, heads, layers, vocab, only=args.design_only))
         for name, cfg in (("llama", llama_at(width, ff, heads, layers, vocab)), (args.design, other)):
             if args.design_skip_llama and name == "llama":
@@ -372,9 +398,10 @@ def main() -> int:
                          "steps of --portion prompt tokens of one request behind --context tokens; 'mixed': such a "
                          "portion beside one decoded token of --batch other requests")
     ap.add_argument("--design-sizes", default="1k,2k", help="design: sizes to run, of " + ",".join(sorted(DESIGN_SIZES)))
-    ap.add_argument("--design", default="rilonex", choices=["rilonex", "bidirax"], help="design: which design runs beside Llama")
-    ap.add_argument("--design-only", default="", choices=["", "rglru", "channel_delta", "parallel", "rotated", "windowed"],
-                    help="design: a model of this kind of layer only (the first three Rilonex, the others Bidirax)")
+    ap.add_argument("--design", default="rilonex", choices=["rilonex", "bidirax", "zetonex"], help="design: which design runs beside Llama")
+    ap.add_argument("--design-only", default="", choices=["", "rglru", "channel_delta", "parallel", "rotated", "windowed", "differential", "gated"],
+                    help="design: a model of this kind of layer only (the first three Rilonex, the next two Bidirax, the last "
+                         "two Zetonex)")
     ap.add_argument("--design-skip-llama", action="store_true", help="design: time the design alone")
     ap.add_argument("--portion", type=int, default=256, help="portion: prompt tokens a step")
     ap.add_argument("--decode-len", type=int, default=700, help="mixed: tokens of the shortest decoding request "
