@@ -28,8 +28,10 @@ namespace llme {
 
 constexpr int kMaxHeadEntries = 256;
 
-// One workgroup per token, a wavefront per head in turn. Rows of p: queries at column 0, keys at k_col, values at
-// v_col (v_col < 0: a value head is the key head as projected, before norm and rotation).
+// A workgroup per (token, group of heads): its four wavefronts take the group's heads in turn (queries first, then
+// keys); gridDim.y groups share a token's heads. The angles of the token's position are made once per workgroup.
+// Rows of p: queries at column 0, keys at k_col, values at v_col (v_col < 0: a value head is the key head as
+// projected, before norm and rotation).
 template <typename TQ, typename TC, typename TW>
 __global__ __launch_bounds__(256) void qk_prepare_kernel(const float* __restrict__ p, int ld, int nq, int nk, int nv, int dk, int dv,
                                                          int k_col, int v_col, const TW* __restrict__ wq, const TW* __restrict__ wk,
@@ -38,6 +40,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(const float* __restrict
                                                          const int* __restrict__ block_table, int max_blocks,
                                                          TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
                                                          int page) {
+    __shared__ float cs_t[kMaxHeadEntries / 2], sn_t[kMaxHeadEntries / 2];
     const int t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int pos = positions[t];
@@ -46,7 +49,14 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(const float* __restrict
     const int pg = block_table[static_cast<size_t>(seq_idx[t]) * max_blocks + pos / page];
     const int in_page = pos % page;
     const int half = rot / 2;
-    for (int u = wave; u < nq + nk; u += 4) {
+    for (int f = threadIdx.x; f < half; f += 256) {
+        float sn, cs;
+        sincosf(fpos * inv_freq[f], &sn, &cs);
+        sn_t[f] = sn;
+        cs_t[f] = cs;
+    }
+    __syncthreads();
+    for (int u = blockIdx.y * 4 + wave; u < nq + nk; u += 4 * gridDim.y) {
         const bool is_q = u < nq;
         const int head = is_q ? u : u - nq;
         const float* hp = row + (is_q ? head * dk : k_col + head * dk);
@@ -64,8 +74,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(const float* __restrict
                 const int f = e < half ? e : e - half;
                 const int pe = e < half ? e + half : e - half;
                 const float other = w != nullptr ? hp[pe] * r * to_float(w[pe]) : hp[pe];
-                float sn, cs;
-                sincosf(fpos * inv_freq[f], &sn, &cs);
+                const float sn = sn_t[f], cs = cs_t[f];
                 v = e < half ? v * cs - other * sn : v * cs + other * sn;
             }
             if (is_q) {
@@ -78,7 +87,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(const float* __restrict
     }
     if (v_col >= 0) {
         const float* vp = row + v_col;
-        for (int e = threadIdx.x; e < nv * dv; e += 256)
+        for (int e = blockIdx.y * 256 + threadIdx.x; e < nv * dv; e += 256 * gridDim.y)
             v_cache[((static_cast<size_t>(pg) * nv + e / dv) * dv + e % dv) * page + in_page] = from_float<TC>(vp[e]);
     }
 }
@@ -200,29 +209,83 @@ __global__ __launch_bounds__(256) void window_attention_finish_kernel(const floa
     if (item >= static_cast<size_t>(T) * heads) return;
     const int t = static_cast<int>(item / heads), head = static_cast<int>(item % heads);
     const int nq = heads * maps;
-    float o[PER_LANE] = {0.f, 0.f, 0.f, 0.f};
-    for (int map = 0; map < maps; ++map) {
-        const size_t at = static_cast<size_t>(t) * nq + head * maps + map;
-        const size_t stride = static_cast<size_t>(T) * nq;
-        float mx = -INFINITY;
-        for (int r = 0; r < runs; ++r) mx = fmaxf(mx, part_ml[(r * stride + at) * 2]);
-        float l = 0.f;
-        float a[PER_LANE] = {0.f, 0.f, 0.f, 0.f};
-        for (int r = 0; r < runs; ++r) {
-            const float mr = part_ml[(r * stride + at) * 2];
-            if (mr == -INFINITY) continue;                  // a run in which the row saw no key
-            const float f = expf(mr - mx);
-            l += f * part_ml[(r * stride + at) * 2 + 1];
+    constexpr int MAPS = MODE == kFinishDifference ? 2 : 1;
+    constexpr int CHUNK = 8;                // runs whose values are asked for together
+    const size_t stride = static_cast<size_t>(T) * nq;
+    const size_t at0 = static_cast<size_t>(t) * nq + head * MAPS;
+    float a[MAPS][PER_LANE], l[MAPS];
+#pragma unroll
+    for (int mp = 0; mp < MAPS; ++mp) {
+        l[mp] = 0.f;
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) a[mp][i] = 0.f;
+    }
+    // lane r holds run r's maximum and sum (64 runs at a time); the runs' values are then added in the order of the
+    // runs, eight runs of every map of the head asked for before the first is used
+    float mx[MAPS];
+#pragma unroll
+    for (int mp = 0; mp < MAPS; ++mp) {
+        float v = -INFINITY;
+        for (int r = lane; r < (runs == 1 ? 0 : runs); r += kWave) v = fmaxf(v, part_ml[(r * stride + at0 + mp) * 2]);
+        mx[mp] = wave_max(v);
+    }
+    if (runs == 1) {                         // (prompts: one run, nothing to join)
+#pragma unroll
+        for (int mp = 0; mp < MAPS; ++mp) {
+            l[mp] = part_ml[(at0 + mp) * 2 + 1];
 #pragma unroll
             for (int i = 0; i < PER_LANE; ++i) {
                 const int d = lane + i * kWave;
-                if (d < dv) a[i] = fmaf(f, part_o[(r * stride + at) * dv + d], a[i]);
+                a[mp][i] = d < dv ? part_o[(at0 + mp) * dv + d] : 0.f;
             }
         }
-        const float inv = 1.0f / l;
-        const float sign = (MODE == kFinishDifference && map == 1) ? -lambda : 1.f;
+    }
+    for (int r0 = 0; r0 < (runs == 1 ? 0 : runs); r0 += kWave) {
+        const int r = r0 + lane;
+        float fr[MAPS], lr[MAPS];
 #pragma unroll
-        for (int i = 0; i < PER_LANE; ++i) o[i] = (MODE == kFinishDifference && map > 0) ? fmaf(sign, a[i] * inv, o[i]) : a[i] * inv;
+        for (int mp = 0; mp < MAPS; ++mp) {
+            fr[mp] = lr[mp] = 0.f;
+            if (r < runs) {
+                const float mr = part_ml[(r * stride + at0 + mp) * 2];
+                fr[mp] = mr == -INFINITY ? 0.f : expf(mr - mx[mp]);            // (a run in which the row saw no key)
+                lr[mp] = part_ml[(r * stride + at0 + mp) * 2 + 1];
+            }
+        }
+        const int n = runs - r0 < kWave ? runs - r0 : kWave;
+        for (int j0 = 0; j0 < n; j0 += CHUNK) {
+            float v[CHUNK][MAPS][PER_LANE];
+#pragma unroll
+            for (int j = 0; j < CHUNK; ++j)
+#pragma unroll
+                for (int mp = 0; mp < MAPS; ++mp)
+#pragma unroll
+                    for (int i = 0; i < PER_LANE; ++i) {
+                        const int d = lane + i * kWave;
+                        v[j][mp][i] = (j0 + j < n && d < dv) ? part_o[((r0 + j0 + j) * stride + at0 + mp) * dv + d] : 0.f;
+                    }
+#pragma unroll
+            for (int j = 0; j < CHUNK; ++j)
+#pragma unroll
+                for (int mp = 0; mp < MAPS; ++mp) {
+                    const int jj = j0 + j < n ? j0 + j : 0;
+                    const float f = j0 + j < n ? __shfl(fr[mp], jj, kWave) : 0.f;
+                    l[mp] = fmaf(f, __shfl(lr[mp], jj, kWave), l[mp]);
+#pragma unroll
+                    for (int i = 0; i < PER_LANE; ++i) a[mp][i] = f != 0.f ? fmaf(f, v[j][mp][i], a[mp][i]) : a[mp][i];
+                }
+        }
+    }
+    float o[PER_LANE];
+    {
+        const float inv = 1.0f / l[0];
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) o[i] = a[0][i] * inv;
+        if (MAPS == 2) {
+            const float inv2 = 1.0f / l[MAPS - 1];
+#pragma unroll
+            for (int i = 0; i < PER_LANE; ++i) o[i] = fmaf(-lambda, a[MAPS - 1][i] * inv2, o[i]);
+        }
     }
     float f = 1.f;
     if (MODE == kFinishDifference) {
@@ -256,8 +319,13 @@ extern "C" int llme_qk_prepare(const float* p, int ld, int nq, int nk, int nv, i
     if (dk <= 0 || dv <= 0 || nv <= 0 || nk % nv != 0 || page <= 0 || rot < 0 || rot > dk || rot % 2 != 0) return kErrBadArgument;
     if ((wq == nullptr) != (wk == nullptr) || (rot > 0 && inv_freq == nullptr)) return kErrBadArgument;
     if (v_col < 0 && (nk != nv || dk != dv)) return kErrBadArgument;
+    if (dk > kMaxHeadEntries) return kErrBadArgument;
+    // enough workgroups for the chip where the step has few tokens: up to a wavefront a head
+    const int head_groups = (nq + nk + 3) / 4;
+    const int want = (2048 + T - 1) / T;
+    const dim3 grid(T, want < head_groups ? (want > 0 ? want : 1) : head_groups);
 #define LLME_PREP(TQ, TC, TW)                                                                                              \
-    hipLaunchKernelGGL((qk_prepare_kernel<TQ, TC, TW>), dim3(T), dim3(256), 0, stream, p, ld, nq, nk, nv, dk, dv, k_col, v_col, \
+    hipLaunchKernelGGL((qk_prepare_kernel<TQ, TC, TW>), grid, dim3(256), 0, stream, p, ld, nq, nk, nv, dk, dv, k_col, v_col, \
                        static_cast<const TW*>(wq), static_cast<const TW*>(wk), eps, inv_freq, rot, positions, seq_idx,    \
                        block_table, max_blocks, static_cast<TQ*>(q_out), static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), page)
     if (q_dtype != cache_dtype) return kErrBadArgument;

@@ -10,11 +10,13 @@
 //
 //   S^T[key, row] = sum_d K[key, d] Q[row, d]     first operand: a key's entries as they lie in its page, 16 bytes a lane
 //   O^T[c, row]  += sum_key V^T[c, key] P^T[key, row]
-// Lane l holds, for query row l % 16, the scores of keys 4 (l / 16) + e of both 16-key halves of a block: exactly the 8
-// keys it supplies as second operand of the second product, so weights never leave their registers. A weight is
-// 32-bit; it enters the second product as the sum of two bfloat16 parts (16 bits of mantissa), and the row's sum adds
-// the 32-bit weights. Operands come straight from the pages (no LDS): the four wavefronts of a workgroup take tiles
-// next to each other and find each other's keys in the cache.
+// The rows of a 16-key half are laid so that lane l ends up, for query row l % 16, with the scores of the 8 consecutive
+// keys 8 (l / 16) .. of the block: exactly the keys it supplies as second operand of the second product (one 16-byte
+// piece of a value row a tile), so weights never leave their registers. A weight is 32-bit; it enters the second
+// product as the sum of two bfloat16 parts (16 bits of mantissa), and the row's sum adds the 32-bit weights. Blocks
+// that every row of the tile sees whole (most of a window) skip the tests of visibility. Operands come straight from
+// the pages (no LDS), the next block's keys asked for while this block's weights are made: the four wavefronts of a
+// workgroup take tiles next to each other and find each other's keys in the cache.
 #include "common.h"
 #include <math.h>
 
@@ -33,9 +35,75 @@ struct WindowArgs {
     const int* positions;
     const int* q_start;
     const int* block_table;
-    int max_blocks, T, nq, nk, nv, maps, per_value_head, dk, dv, page, window, keep_first, nsplit;
+    int max_blocks, T, nq, nk, nv, maps, per_value_head, dk, dv, page, page_shift, window, keep_first, nsplit;
     float scale, softcap;
 };
+
+// tanh for the capped scores: the odd series where |y| is small (there 1 - 2 / (e^2y + 1) would cancel), the
+// exponential elsewhere; both in 32-bit with the hardware's exponential and reciprocal.
+__device__ __forceinline__ float cap_tanh(float y) {
+    const float y2 = y * y;
+    const float series = y * (1.f + y2 * (-1.f / 3.f + y2 * (2.f / 15.f)));
+    const float e = __expf(2.f * y);
+    const float wide = 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
+    return fabsf(y) < 0.05f ? series : wide;
+}
+
+// One block of 32 keys for a tile: scores in sc (this lane's row, keys key0 + 8 qd + j for j = 4 sub + e), values in vf.
+// EDGE: some row of the tile does not see some key of the block (the window's start, the diagonal, kept tokens, rows
+// beyond the request), or a key lies behind the tile's last; otherwise every weight counts and no test is made.
+template <int NVM, bool EDGE, bool CAP>
+__device__ __forceinline__ void window_block(const WindowArgs& a, const f32x4 (&sc)[2], bf16x8 (&vf)[NVM], f32x4 (&acc)[NVM], float& m,
+                                             float& l, int nvt, int key0, int qd, int pos, int pos_max, bool valid, float inv_cap) {
+    float p[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        float v = sc[j >> 2][j & 3] * a.scale;
+        if (CAP) v = a.softcap * cap_tanh(v * inv_cap);
+        if (EDGE) {
+            const int key = key0 + qd * 8 + j;
+            const bool seen = valid && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
+            v = seen ? v : -INFINITY;
+        }
+        p[j] = v;
+        mx = fmaxf(mx, v);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = (EDGE && m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __expf(m - m_use);
+    m = m_new;
+    float sum = 0.f;
+    bf16x8 ph, pl;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float w = __expf(p[j] - m_use);
+        sum += w;
+        const bf16 hi = static_cast<bf16>(w);
+        ph[j] = hi;
+        pl[j] = static_cast<bf16>(w - static_cast<float>(hi));
+    }
+    l = l * alpha + sum;
+#pragma unroll
+    for (int c = 0; c < NVM; ++c) {
+        if (c < nvt) {
+            bf16x8 v = vf[c];
+            if (EDGE) {
+                // a value behind the tile's last key may be anything that a freed page holds: its weight is zero, and
+                // so is the value the product sees
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (key0 + qd * 8 + j > pos_max) v[j] = static_cast<bf16>(0.f);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[c][e] *= alpha;
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, ph, acc[c], 0, 0, 0);
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pl, acc[c], 0, 0, 0);
+        }
+    }
+}
 
 template <int DSM, int NVM>     // 32-entry slabs of a key, 16-entry tiles of a value: the most this instance holds
 __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WindowArgs a) {
@@ -48,15 +116,18 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WindowArgs a
     const int R0 = (blockIdx.x * 4 + wave) * 16;
     if (R0 >= rows_total) return;
     const bool valid = R0 + r < rows_total;
+    const bool all_valid = R0 + 15 < rows_total;
     const int R = valid ? R0 + r : rows_total - 1;
     const int t = row0 + R / a.per_value_head;
     const int qh = (vh * a.per_value_head + R % a.per_value_head) * a.maps + map;
     const int pos = a.positions[t];
     const int pos_min = a.positions[row0 + R0 / a.per_value_head];
-    const int last_row = R0 + 15 < rows_total ? R0 + 15 : rows_total - 1;
+    const int last_row = all_valid ? R0 + 15 : rows_total - 1;
     const int pos_max = a.positions[row0 + last_row / a.per_value_head];
     const int* table = a.block_table + static_cast<size_t>(s) * a.max_blocks;
     const int ds = (a.dk + 31) >> 5, nvt = a.dv >> 4;
+    const int psh = a.page_shift, pmask = a.page - 1;
+    const float inv_cap = a.softcap > 0.f ? 1.0f / a.softcap : 0.f;
 
     bf16x8 qf[DSM];
     {
@@ -91,103 +162,62 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WindowArgs a
 #pragma unroll
     for (int c = 0; c < NVM; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    for (int b = b_begin; b < b_end; ++b) {
+    // Row i of a 16-key half `sub` of a block is key 8 (i / 4) + 4 sub + i % 4, so that the lane that ends up with rows
+    // 4 qd .. 4 qd + 3 of both halves holds the 8 consecutive keys 8 qd .. 8 qd + 7: one 16-byte piece of a value row.
+    const int k_in_block = 8 * (r >> 2) + (r & 3);
+    bf16x8 kf[2][DSM];
+    auto load_keys = [&](int b) {
         const int key0 = (b < nb_kept ? b : first_blk + b - nb_kept) << 5;
-        f32x4 sc[2];
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
-            int key = key0 + sub * 16 + r;
+            int key = key0 + k_in_block + 4 * sub;
             key = key < pos_max ? key : pos_max;               // (keys behind the tile's last are masked below)
-            int pg = table[key / a.page];
+            int pg = table[key >> psh];
             pg = pg < 0 ? 0 : pg;           // (a page that the window has left behind and given back: its keys are masked)
-            const bf16* krow = a.k_cache + ((static_cast<size_t>(pg) * a.nk + kh) * a.page + key % a.page) * a.dk;
-            sc[sub] = f32x4{0.f, 0.f, 0.f, 0.f};
+            const bf16* krow = a.k_cache + (((static_cast<size_t>(pg) * a.nk + kh) << psh) + (key & pmask)) * a.dk;
 #pragma unroll
             for (int c = 0; c < DSM; ++c) {
                 const int d0 = c * 32 + qd * 8;
-                if (c < ds) {
-                    bf16x8 kf;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) kf[e] = static_cast<bf16>(0.f);
-                    if (d0 < a.dk) kf = *reinterpret_cast<const bf16x8*>(krow + d0);
-                    sc[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], sc[sub], 0, 0, 0);
-                }
+                for (int e = 0; e < 8; ++e) kf[sub][c][e] = static_cast<bf16>(0.f);
+                if (c < ds && d0 < a.dk) kf[sub][c] = *reinterpret_cast<const bf16x8*>(krow + d0);
             }
         }
-        // the values of this lane's 8 keys for every tile of value entries: asked for before the softmax
+    };
+    if (b_begin < b_end) load_keys(b_begin);
+
+    for (int b = b_begin; b < b_end; ++b) {
+        const int key0 = (b < nb_kept ? b : first_blk + b - nb_kept) << 5;
+        // the values of this lane's 8 keys for every tile of value entries: asked for before the scores are made
         bf16x8 vf[NVM];
         {
-            int kq[2], pgs[2];
+            const int kq = key0 + qd * 8;
+            const int kc = kq <= pos_max ? kq : (pos_max & ~7);
+            int pg = table[kc >> psh];
+            pg = pg < 0 ? 0 : pg;
+            const bf16* vbase = a.v_cache + ((static_cast<size_t>(pg) * a.nv + vh) * a.dv << psh) + (kc & pmask);
 #pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-                kq[sub] = key0 + sub * 16 + qd * 4;
-                const int kc = kq[sub] <= pos_max ? kq[sub] : (pos_max & ~3);
-                pgs[sub] = table[kc / a.page];
-                pgs[sub] = pgs[sub] < 0 ? 0 : pgs[sub];
-                kq[sub] = kc;
-            }
-#pragma unroll
-            for (int c = 0; c < NVM; ++c) {
-                if (c < nvt) {
-                    const int ch = c * 16 + r;
-#pragma unroll
-                    for (int sub = 0; sub < 2; ++sub) {
-                        const bf16* vp = a.v_cache + ((static_cast<size_t>(pgs[sub]) * a.nv + vh) * a.dv + ch) * a.page + kq[sub] % a.page;
-                        const bf16x4 v4 = *reinterpret_cast<const bf16x4*>(vp);
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) vf[c][sub * 4 + e] = v4[e];
-                    }
-                }
-            }
+            for (int c = 0; c < NVM; ++c)
+                if (c < nvt) vf[c] = *reinterpret_cast<const bf16x8*>(vbase + (static_cast<size_t>(c * 16 + r) << psh));
         }
-        float p[8];
-        float mx = -INFINITY;
+        f32x4 sc[2];
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
+            sc[sub] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int key = key0 + sub * 16 + qd * 4 + e;
-                float v = sc[sub][e] * a.scale;
-                if (a.softcap > 0.f) v = a.softcap * tanhf(v / a.softcap);
-                const bool seen = valid && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
-                v = seen ? v : -INFINITY;
-                p[sub * 4 + e] = v;
-                mx = fmaxf(mx, v);
-            }
+            for (int c = 0; c < DSM; ++c)
+                if (c < ds) sc[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[sub][c], qf[c], sc[sub], 0, 0, 0);
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m, mx);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = expf(m - m_use);
-        m = m_new;
-        float sum = 0.f;
-        bf16x8 ph, pl;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float w = expf(p[e] - m_use);
-            sum += w;
-            const bf16 hi = static_cast<bf16>(w);
-            ph[e] = hi;
-            pl[e] = static_cast<bf16>(w - static_cast<float>(hi));
-        }
-        l = l * alpha + sum;
-#pragma unroll
-        for (int c = 0; c < NVM; ++c) {
-            if (c < nvt) {
-                // a value behind the tile's last key may be anything that a freed page holds: its weight is zero, and
-                // so is the value the product sees
-                bf16x8 v = vf[c];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int key = key0 + (e >> 2) * 16 + qd * 4 + (e & 3);
-                    if (key > pos_max) v[e] = static_cast<bf16>(0.f);
-                }
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc[c][e] *= alpha;
-                acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, ph, acc[c], 0, 0, 0);
-                acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pl, acc[c], 0, 0, 0);
-            }
+        if (b + 1 < b_end) load_keys(b + 1);                    // the next block's keys travel while this one's weights are made
+        // every row sees every key of the block: behind the window's start of the tile's last row, up to the tile's
+        // first position, not among the kept blocks (whose keys may lie beyond keep_first)
+        const bool inner = all_valid && b >= nb_kept && key0 + 31 <= pos_min && (a.window <= 0 || pos_max - key0 < a.window);
+        if (a.softcap > 0.f) {
+            if (inner) window_block<NVM, false, true>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
+            else window_block<NVM, true, true>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
+        } else {
+            if (inner) window_block<NVM, false, false>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
+            else window_block<NVM, true, false>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
         }
     }
     l += __shfl_xor(l, 16, 64);
@@ -208,15 +238,15 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WindowArgs a
 using namespace llme;
 
 // max_new: the most tokens a request brings to the step (sizes the grid). Refuses (10002) what the kernel does not
-// take: key entries no multiple of 8 or beyond 128, value entries no multiple of 16 or beyond 128, pages no multiple
-// of 16.
+// take: key entries no multiple of 8 or beyond 128, value entries no multiple of 16 or beyond 128, pages that are no
+// power of two from 16 on.
 extern "C" int llme_window_attention_mfma(const void* q, const void* k_cache, const void* v_cache, float* part_o, float* part_ml,
                                           const int* positions, const int* q_start, const int* block_table, int max_blocks, int T,
                                           int S, int max_new, int nq, int nk, int nv, int dk, int dv, int page, float scale,
                                           float softcap, int window, int keep_first, int nsplit, hipStream_t stream) {
     if (T <= 0 || S <= 0) return 0;
     if (nv <= 0 || nk % nv != 0 || nq % nk != 0 || max_new <= 0 || nsplit <= 0 || window < 0 || keep_first < 0) return kErrBadArgument;
-    if (dk % 8 != 0 || dk > 128 || dv % 16 != 0 || dv > 128 || page % 16 != 0) return kErrUnsupported;
+    if (dk % 8 != 0 || dk > 128 || dv % 16 != 0 || dv > 128 || page % 16 != 0 || (page & (page - 1)) != 0) return kErrUnsupported;
     WindowArgs a;
     a.q = static_cast<const bf16*>(q);
     a.k_cache = static_cast<const bf16*>(k_cache);
@@ -236,6 +266,7 @@ extern "C" int llme_window_attention_mfma(const void* q, const void* k_cache, co
     a.dk = dk;
     a.dv = dv;
     a.page = page;
+    a.page_shift = __builtin_ctz(page);
     a.window = window;
     a.keep_first = keep_first;
     a.nsplit = nsplit;
