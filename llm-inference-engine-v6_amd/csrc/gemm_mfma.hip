@@ -52,15 +52,38 @@ typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 constexpr int kBufferFlags = 0x00020000;
 
 enum OutMode : int { kStoreF32 = 0, kAddF32 = 1, kStoreBF16 = 2, kAtomicF32 = 3, kGatedBF16 = 4, kRopeCache = 5,
-                     kGatedReluBF16 = 6, kGatedGeluBF16 = 7 };
+                     kGatedReluBF16 = 6, kGatedGeluBF16 = 7, kGatedExtraBF16 = 8 };
 // The gated outputs: act(gate) * up with act = SiLU (kGatedBF16), the rectifier (kGatedReluBF16) or the tanh form of
-// GELU (kGatedGeluBF16).
-constexpr bool is_gated(int mode) { return mode == kGatedBF16 || mode == kGatedReluBF16 || mode == kGatedGeluBF16; }
+// GELU (kGatedGeluBF16); kGatedExtraBF16: SiLU or a clamped swish with biases on gate and up (GateExtra).
+constexpr bool is_gated(int mode) {
+    return mode == kGatedBF16 || mode == kGatedReluBF16 || mode == kGatedGeluBF16 || mode == kGatedExtraBF16;
+}
 template <int MODE> __device__ __forceinline__ float gate_act(float g) {
     if (MODE == kGatedReluBF16) return fmaxf(g, 0.f);
     if (MODE == kGatedGeluBF16) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
     return g / (1.0f + expf(-g));
 }
+// What kGatedExtraBF16 does around the activation. bias [N] in the order of w's rows (so in the order of the product's
+// columns): added to gate and up first. limit > 0: gate <- min(gate, limit), up <- clamp(up, -limit, limit) and the
+// value is gate sigmoid(alpha gate) (up + 1); otherwise silu(gate) up.
+struct GateExtra {
+    const bf16* bias = nullptr;
+    float limit = 0.f, alpha = 1.f;
+};
+// bg, bu: the biases of this gate and up value (zero where there are none).
+template <int MODE> __device__ __forceinline__ float gated_value(float g, float u, const GateExtra& gx, float bg, float bu) {
+    if (MODE != kGatedExtraBF16) return gate_act<MODE>(g) * u;
+    g += bg;
+    u += bu;
+    if (gx.limit > 0.f) {
+        g = fminf(g, gx.limit);
+        u = fminf(fmaxf(u, -gx.limit), gx.limit);
+        return g / (1.0f + expf(-gx.alpha * g)) * (u + 1.0f);
+    }
+    return g / (1.0f + expf(-g)) * u;
+}
+// The extras of the launches that an entry point is making (set and cleared inside one call, on the caller's thread).
+static thread_local GateExtra t_gate_extra;
 
 // Products in groups (the tile kernel's GROUPED instances): every row tile belongs to one group and is multiplied by that
 // group's matrix, w + group * w_stride.
@@ -154,7 +177,7 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
                                               int M, int N, int m0, int n0, int wm, int wn, int tid, int r, int q,
                                               const QkvTarget& qt = QkvTarget{},
                                               const AddendsAhead<WR * 16 * WMT, WC * 16 * WNT, 64 * WR * WC>& ahead = {},
-                                              const RowPlace& place = RowPlace{}) {
+                                              const RowPlace& place = RowPlace{}, const GateExtra& gx = GateExtra{}) {
     constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT, NT = 64 * WR * WC;
 
     constexpr int SS = BN + 4;                           // floats per staged row
@@ -269,11 +292,15 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
                 const int m = mp + row, n = n0 + col;
                 if (m >= M || n >= N) continue;
                 const float* gp = stage + row * SS + col;
-                bf16x8 o;
+                bf16x8 o, bgv = zero8(), buv = zero8();
+                if (MODE == kGatedExtraBF16 && gx.bias != nullptr) {    // (a piece's gates are columns n .., its ups 16 on)
+                    bgv = *reinterpret_cast<const bf16x8*>(gx.bias + n);
+                    buv = *reinterpret_cast<const bf16x8*>(gx.bias + n + 16);
+                }
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float gt = gp[e], up = gp[16 + e];
-                    o[e] = static_cast<__bf16>(gate_act<MODE>(gt) * up);
+                    o[e] = static_cast<__bf16>(gated_value<MODE>(gt, up, gx, static_cast<float>(bgv[e]), static_cast<float>(buv[e])));
                 }
                 const int unit = (n0 + (piece / 2) * 32) / 2 + (piece % 2) * 8;
                 *reinterpret_cast<bf16x8*>(static_cast<bf16*>(out) + static_cast<size_t>(m) * (N / 2) + unit) = o;
@@ -338,8 +365,13 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
                     const int unit = (n0 + wn + j * 16) / 2 + r;        // tile column pair (gate, up)
                     if (2 * unit >= N) continue;
                     const float gt = acc[i][j][e], up = acc[i][j + 1][e];
+                    float bg = 0.f, bu = 0.f;
+                    if (MODE == kGatedExtraBF16 && gx.bias != nullptr) {
+                        bg = static_cast<float>(gx.bias[n0 + wn + j * 16 + r]);
+                        bu = static_cast<float>(gx.bias[n0 + wn + j * 16 + r + 16]);
+                    }
                     static_cast<bf16*>(out)[static_cast<size_t>(m) * (N / 2) + unit] =
-                        static_cast<bf16>(gate_act<MODE>(gt) * up);
+                        static_cast<bf16>(gated_value<MODE>(gt, up, gx, bg, bu));
                 }
             } else {
 #pragma unroll
@@ -364,7 +396,7 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
 template <int WMT, int WNT, int MODE, bool KFULL, bool BLOCKED, bool GROUPED = false>
 __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w,
                                                         void* __restrict__ out, int M, int N, int K,
-                                                        int tiles_m, int tiles_n, int ksplit, QkvTarget qt, Groups gr) {
+                                                        int tiles_m, int tiles_n, int ksplit, QkvTarget qt, Groups gr, GateExtra gx) {
     constexpr int BM = 32 * WMT, BN = 32 * WNT;
     constexpr int A_ELEMS = BM * TSTRIDE, W_ELEMS = BN * TSTRIDE;
     constexpr int CA = BM / 32, CW = BN / 32;        // 16-byte chunks per thread and slab
@@ -586,7 +618,7 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
     if (AHEAD && N % 8 == 0) addends.load(out, M, N, m0, n0, tid);
     __syncthreads();                                  // the epilogue reuses the slabs' LDS
     tile_epilogue<WMT, WNT, MODE, tile_lds_bytes<WMT, WNT>(), 2, 2, AHEAD>(acc, lds_raw, out, M, N, m0, n0, wm, wn, tid, r, q,
-                                                                           qt, addends, place);
+                                                                           qt, addends, place, gx);
 }
 
 // ----------------------------------------------------------------------------------------
@@ -643,7 +675,7 @@ __device__ __forceinline__ void load_b128_to_lds(u32x4 rsrc, unsigned lds_base, 
 template <int WR, int WC, int WMT, int WNT, int MODE>
 __global__ __launch_bounds__(64 * WR * WC, 1) void gemm_tile_direct_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, void* __restrict__ out, int M, int N, int K, int tiles_m,
-    int tiles_n, int ksplit, QkvTarget qt, Groups) {        // (no grouped instances: the argument keeps the launches alike)
+    int tiles_n, int ksplit, QkvTarget qt, Groups, GateExtra gx) {  // (no grouped instances: the argument keeps the launches alike)
     constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT, NW = WR * WC;
     constexpr int AC = BM / 8, WB = BN / 16;                    // loads: chunks of a slab of A, blocks of half a slab of W
     static_assert(AC % NW == 0 && WB % NW == 0, "every wavefront has the same loads");
@@ -777,7 +809,7 @@ __global__ __launch_bounds__(64 * WR * WC, 1) void gemm_tile_direct_kernel(
     }
     wait_vm<0>();                                       // (loads past the end are still on their way into LDS)
     __syncthreads();                                    // the epilogue reuses the slabs' LDS
-    tile_epilogue<WMT, WNT, MODE, 160 * 1024, WR, WC>(acc, lds_raw, out, M, N, m0, n0, wm, wn, tid, r, q, qt);
+    tile_epilogue<WMT, WNT, MODE, 160 * 1024, WR, WC>(acc, lds_raw, out, M, N, m0, n0, wm, wn, tid, r, q, qt, {}, RowPlace{}, gx);
 }
 
 template <auto KERNEL, int THREADS = 256>
@@ -792,7 +824,7 @@ static int launch_tile_kernel(int LDS, int BM, int BN, const bf16* A, const bf16
     }
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(KERNEL, dim3(tiles_m * tiles_n * ksplit), dim3(THREADS), LDS, stream, A, W, out, M, N, K, tiles_m,
-                       tiles_n, ksplit, qt, Groups{});
+                       tiles_n, ksplit, qt, Groups{}, t_gate_extra);
     return launch_status();
 }
 
@@ -810,7 +842,7 @@ static int launch_grouped_mode(const bf16* A, const bf16* W, void* out, int M, i
             attr_set = true;
         }
         hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(256), LDS, stream, A, W, out, M, N, K, tiles_m, tiles_n, 1,
-                           QkvTarget{}, gr);
+                           QkvTarget{}, gr, t_gate_extra);
         return launch_status();
     };
     if (K % TK != 0) return go(&gemm_tile_kernel<WMT, WNT, MODE, false, false, true>);
@@ -822,6 +854,7 @@ static int launch_grouped(const bf16* A, const bf16* W, void* out, int M, int N,
     switch (mode) {
         case kStoreF32: return launch_grouped_mode<WMT, WNT, kStoreF32>(A, W, out, M, N, K, tiles_m, gr, stream);
         case kGatedBF16: return launch_grouped_mode<WMT, WNT, kGatedBF16>(A, W, out, M, N, K, tiles_m, gr, stream);
+        case kGatedExtraBF16: return launch_grouped_mode<WMT, WNT, kGatedExtraBF16>(A, W, out, M, N, K, tiles_m, gr, stream);
         case kStoreBF16: return launch_grouped_mode<WMT, WNT, kStoreBF16>(A, W, out, M, N, K, tiles_m, gr, stream);
         default: return kErrBadArgument;
     }
@@ -855,6 +888,7 @@ static int launch_tile(const bf16* A, const bf16* W, void* out, int M, int N, in
         case kGatedBF16: return launch_tile_mode<WMT, WNT, kGatedBF16>(A, W, out, M, N, K, 1, blocked, stream);
         case kGatedReluBF16: return launch_tile_mode<WMT, WNT, kGatedReluBF16>(A, W, out, M, N, K, 1, blocked, stream);
         case kGatedGeluBF16: return launch_tile_mode<WMT, WNT, kGatedGeluBF16>(A, W, out, M, N, K, 1, blocked, stream);
+        case kGatedExtraBF16: return launch_tile_mode<WMT, WNT, kGatedExtraBF16>(A, W, out, M, N, K, 1, blocked, stream);
         default: return launch_tile_mode<WMT, WNT, kStoreBF16>(A, W, out, M, N, K, 1, blocked, stream);
     }
 }
@@ -874,6 +908,7 @@ static int launch_tile_direct(const bf16* A, const bf16* W, void* out, int M, in
         case kGatedBF16: return LLME_DIRECT(kGatedBF16);
         case kGatedReluBF16: return LLME_DIRECT(kGatedReluBF16);
         case kGatedGeluBF16: return LLME_DIRECT(kGatedGeluBF16);
+        case kGatedExtraBF16: return LLME_DIRECT(kGatedExtraBF16);
         default: return LLME_DIRECT(kStoreBF16);
     }
 #undef LLME_DIRECT
@@ -1065,7 +1100,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     // tile shape: 0 lets the entry point choose: the largest tile that still gives about one
     // workgroup per compute unit; a small output with a long k is cut over k instead (the
     // parts are added with atomics, so this needs an accumulating float32 output).
-    if (gated) mode = gated == 2 ? kGatedReluBF16 : gated == 3 ? kGatedGeluBF16 : kGatedBF16;
+    if (gated) mode = gated == 2 ? kGatedReluBF16 : gated == 3 ? kGatedGeluBF16 : gated == 4 ? kGatedExtraBF16 : kGatedBF16;
     const bool auto_shape = tile_shape <= 0;
     float tiles_cost = -1.f;                           // of the chosen tile, in the units of the estimate below
     if (tile_shape <= 0) {
@@ -1199,11 +1234,38 @@ extern "C" int llme_gemm_bf16_grouped(const void* a, const void* w, void* out, i
         tiles_m = groups * gr.tiles_per_group;
         M = groups * rows_per_group;
     }
-    const int mode = gated ? kGatedBF16 : out_dtype == kBF16 ? kStoreBF16 : kStoreF32;
+    const int mode = gated == 4 ? kGatedExtraBF16 : gated ? kGatedBF16 : out_dtype == kBF16 ? kStoreBF16 : kStoreF32;
     const bf16* A = static_cast<const bf16*>(a);
     const bf16* W = static_cast<const bf16*>(w);
     if (tile == 128) return launch_grouped<4, 4>(A, W, out, M, N, K, mode, tiles_m, gr, stream);
     return launch_grouped<2, 2>(A, W, out, M, N, K, mode, tiles_m, gr, stream);
+}
+
+// The gated products with what GateExtra names around the activation: bias [N] bfloat16 in the order of w's rows (or
+// null), limit > 0 for the clamped swish with its alpha (limit 0: SiLU). Otherwise llme_gemm_bf16 with gated set.
+extern "C" int llme_gemm_bf16_gated_extra(const void* a, const void* w, void* out, int M, int N, int K, const void* bias, float limit,
+                                          float alpha, int tile_shape, int blocked, int direct, hipStream_t stream) {
+    if (limit < 0.f) return kErrBadArgument;
+    t_gate_extra.bias = static_cast<const bf16*>(bias);
+    t_gate_extra.limit = limit;
+    t_gate_extra.alpha = alpha;
+    const int rc = llme_gemm_bf16(a, w, out, kBF16, M, N, K, 0, 4, 0, 0, tile_shape, blocked, direct, stream);
+    t_gate_extra = GateExtra{};
+    return rc;
+}
+
+// The experts' gate/up product (llme_gemm_bf16_grouped with tile_group given) with the clamped swish; experts have no biases.
+extern "C" int llme_gemm_bf16_grouped_gated_extra(const void* a, const void* w, void* out, int N, int K, int tile, int max_tiles,
+                                                  const int* tile_group, const int* n_tiles, const int* row_index, int gather_div,
+                                                  long a_rows, int groups, float limit, float alpha, hipStream_t stream) {
+    if (limit < 0.f || tile_group == nullptr) return kErrBadArgument;
+    t_gate_extra.bias = nullptr;
+    t_gate_extra.limit = limit;
+    t_gate_extra.alpha = alpha;
+    const int rc = llme_gemm_bf16_grouped(a, w, out, kBF16, 4, N, K, tile, max_tiles, tile_group, n_tiles, row_index, gather_div,
+                                          a_rows, groups, 0, stream);
+    t_gate_extra = GateExtra{};
+    return rc;
 }
 
 // The q/k/v projection of many rows (prompts) with rotation and cache write in its epilogue:

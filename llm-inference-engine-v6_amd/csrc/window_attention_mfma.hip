@@ -73,7 +73,9 @@ __device__ __forceinline__ void window_block(const WindowArgs& a, const f32x4 (&
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m, mx);
     const float m_use = (EDGE && m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __expf(m - m_use);
+    // (where no row of the tile has a new maximum, which is the rule behind the first blocks, alpha is 1 for all)
+    const bool rescale = __any(m_new != m);
+    const float alpha = rescale ? __expf(m - m_use) : 1.f;
     m = m_new;
     float sum = 0.f;
     bf16x8 ph, pl;
@@ -85,7 +87,7 @@ __device__ __forceinline__ void window_block(const WindowArgs& a, const f32x4 (&
         ph[j] = hi;
         pl[j] = static_cast<bf16>(w - static_cast<float>(hi));
     }
-    l = l * alpha + sum;
+    l = rescale ? l * alpha + sum : l + sum;
 #pragma unroll
     for (int c = 0; c < NVM; ++c) {
         if (c < nvt) {
@@ -97,16 +99,19 @@ __device__ __forceinline__ void window_block(const WindowArgs& a, const f32x4 (&
                 for (int j = 0; j < 8; ++j)
                     if (key0 + qd * 8 + j > pos_max) v[j] = static_cast<bf16>(0.f);
             }
+            if (rescale) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[c][e] *= alpha;
+                for (int e = 0; e < 4; ++e) acc[c][e] *= alpha;
+            }
             acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, ph, acc[c], 0, 0, 0);
             acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pl, acc[c], 0, 0, 0);
         }
     }
 }
 
-template <int DSM, int NVM>     // 32-entry slabs of a key, 16-entry tiles of a value: the most this instance holds
-__global__ __launch_bounds__(256) void window_attention_mfma_kernel(WindowArgs a) {
+// DSM, NVM: 32-entry slabs of a key, 16-entry tiles of a value: the most this instance holds. CAP: scores are capped.
+template <int DSM, int NVM, bool CAP>
+__global__ __launch_bounds__(256, (DSM <= 2 && NVM <= 4) ? 4 : NVM <= 4 ? 3 : 2) void window_attention_mfma_kernel(WindowArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, qd = lane >> 4;
     const int s = blockIdx.y / a.nk, kh = blockIdx.y % a.nk;
@@ -212,13 +217,8 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WindowArgs a
         // every row sees every key of the block: behind the window's start of the tile's last row, up to the tile's
         // first position, not among the kept blocks (whose keys may lie beyond keep_first)
         const bool inner = all_valid && b >= nb_kept && key0 + 31 <= pos_min && (a.window <= 0 || pos_max - key0 < a.window);
-        if (a.softcap > 0.f) {
-            if (inner) window_block<NVM, false, true>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
-            else window_block<NVM, true, true>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
-        } else {
-            if (inner) window_block<NVM, false, false>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
-            else window_block<NVM, true, false>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
-        }
+        if (inner) window_block<NVM, false, CAP>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
+        else window_block<NVM, true, CAP>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
     }
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -274,7 +274,11 @@ extern "C" int llme_window_attention_mfma(const void* q, const void* k_cache, co
     a.softcap = softcap;
     const int tiles = (max_new * a.per_value_head + 15) / 16;
     const dim3 grid((tiles + 3) / 4, S * nk, nsplit);
-#define LLME_WMFMA(DSM, NVM) hipLaunchKernelGGL((window_attention_mfma_kernel<DSM, NVM>), grid, dim3(256), 0, stream, a)
+#define LLME_WMFMA(DSM, NVM)                                                                                     \
+    do {                                                                                                         \
+        if (softcap > 0.f) hipLaunchKernelGGL((window_attention_mfma_kernel<DSM, NVM, true>), grid, dim3(256), 0, stream, a); \
+        else hipLaunchKernelGGL((window_attention_mfma_kernel<DSM, NVM, false>), grid, dim3(256), 0, stream, a);  \
+    } while (0)
     if (dk <= 64 && dv <= 64) LLME_WMFMA(2, 4);
     else if (dk <= 64) LLME_WMFMA(2, 8);
     else if (dv <= 64) LLME_WMFMA(4, 4);

@@ -80,6 +80,34 @@ def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, grou
         gated_activation(gu, out, group, activation)
 
 
+declare("llme_gemm_bf16_gated_extra", [_vp, _vp, _vp, _i, _i, _i, _vp, _f, _f, _i, _i, _i, _vp])
+GATED_EXTRA_MIN_ROWS = 17       # fewer rows (decoded tokens) go through the skinny product and the activation kernel
+
+
+def gemm_gated_extra(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, group: int, bias: torch.Tensor | None = None,
+                     limit: float = 0.0, alpha: float = 1.0, choices: KernelChoices | None = None) -> bool:
+    """out [T, FF] = act(x Wg^T + bg) * (x Wu^T + bu) in the tile kernels' epilogue, where that fits (returns False where
+    not, and nothing is done): gate and up rows interleaved in groups of 16 in w_gate_up [2 FF, K], bias [2 FF] bfloat16 in
+    the same order or None; limit 0: act is SiLU; limit > 0: g = min(gate, limit), u = clamp(up, -limit, limit) and the
+    value is g sigmoid(alpha g) (u + 1)."""
+    T, FF = out.shape
+    if not ((choices or DEFAULT).fast_gemm and group == 16 and T >= GATED_EXTRA_MIN_ROWS and out.dtype == torch.bfloat16
+            and (2 * FF) % 32 == 0 and x.dtype == torch.bfloat16 and gemm_bf16_supported(x, w_gate_up, out, False)):
+        return False
+    if bias is not None and not (bias.is_cuda and bias.dtype == torch.bfloat16 and tuple(bias.shape) == (2 * FF,)
+                                 and bias.is_contiguous() and bias.data_ptr() % 16 == 0):
+        return False
+    require(x, "x", torch.bfloat16, (T, None))
+    K = x.shape[1]
+    N, _ = kernels._require_weight(w_gate_up, "w_gate_up", torch.bfloat16, K)
+    if N != 2 * FF or limit < 0:
+        raise kernels.KernelError(f"gemm_gated_extra: {N} weight rows for {FF} units, limit {limit}")
+    check(entry("llme_gemm_bf16_gated_extra")(ptr(x), ptr(w_gate_up), ptr(out), T, N, K, ptr(bias) if bias is not None else None,
+                                              float(limit), float(alpha), 0, 1 if kernels.is_blocked(w_gate_up) else 0, -1, stream()),
+          "gemm_gated_extra")
+    return True
+
+
 declare("llme_gemm_bf16_qkv_rope", [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])
 
 

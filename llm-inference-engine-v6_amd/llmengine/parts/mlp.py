@@ -74,11 +74,13 @@ class GatedMLP(FeedForward):
             weight, eps = pre_norm.fused_rms()
             ops.gemv_norm(x, weight, eps, self.w_gate_up, act, gated=True)
         elif self.bias:
-            # the product's 32-bit rows, then biases and activation in one pass
             act = step.buffer("mlp.act", (T, FF), x.dtype)
-            gu = step.buffer("mlp.gate_up", (T, 2 * FF), torch.float32)
-            ops.gemm(x, self.w_gate_up, gu, choices=step.choices)
-            ops.window.gated_bias_act(gu, act, self.group, self.activation, self.b_gate_up)
+            if self.activation != "silu" or not ops.gemm_gated_extra(x, self.w_gate_up, act, self.group, self.b_gate_up,
+                                                                    choices=step.choices):
+                # (few rows, or another type or activation) the product's 32-bit rows, then biases and activation in one pass
+                gu = step.buffer("mlp.gate_up", (T, 2 * FF), torch.float32)
+                ops.gemm(x, self.w_gate_up, gu, choices=step.choices)
+                ops.window.gated_bias_act(gu, act, self.group, self.activation, self.b_gate_up)
         else:
             act = step.buffer("mlp.act", (T, FF), x.dtype)
             ops.gemm_gated(x, self.w_gate_up, act, self.group,

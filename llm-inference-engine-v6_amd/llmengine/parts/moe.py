@@ -102,7 +102,11 @@ class MixtureOfExperts(FeedForward):
         tile_expert, n_tiles = step.buffer("moe.tile_expert", (cap // tile,), i32), step.buffer("moe.tiles", (1,), i32)
         ops.moe_plan(ids, E, tile, place_pair, pair_place, tile_expert, n_tiles)
         act = step.buffer("moe.act", (cap, FF), step.act_dtype)
-        if self.activation == "swish_clamped":
+        if self.activation == "swish_clamped" and ops.latent.moe_gemm_clamped(x, self.w_gate_up, self.group, act, place_pair,
+                                                                             tile_expert, n_tiles, tile, top, self.limit, 1.702,
+                                                                             step.choices):
+            pass                            # (clamps and activation in the product's epilogue)
+        elif self.activation == "swish_clamped":
             # the gate and up columns as 32-bit rows, then clamps and activation in one pass
             gu = step.buffer("moe.gate_up", (cap, 2 * FF), f32)
             ops.moe_gemm(x, self.w_gate_up, False, 0, gu, place_pair, tile_expert, n_tiles, tile, top, "silu", step.choices)

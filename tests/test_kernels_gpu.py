@@ -349,6 +349,44 @@ def test_gemm_gated(ops, T, FF, K, tile):
     assert _rel(out2.cpu().double(), ref) < 5e-3
 
 
+@pytest.mark.parametrize("T,FF,K,bias,limit,blocked", [(17, 176, 64, True, 0.0, False), (130, 256, 96, True, 0.0, True),
+                                                       (300, 208, 160, False, 1.5, True), (2048, 4096, 1024, True, 0.0, True),
+                                                       (273, 352, 72, True, 2.0, False), (64, 2048, 512, False, 0.75, True)])
+def test_gemm_gated_with_biases_and_clamps(ops, T, FF, K, bias, limit, blocked):
+    """The gated product whose epilogue adds biases to gate and up and applies SiLU, or the clamped swish
+    g sigmoid(alpha g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit), against the formula in 64-bit."""
+    x = torch.randn(T, K, generator=_gen(133)).to(torch.bfloat16)
+    wg = (0.2 * torch.randn(FF, K, generator=_gen(134))).to(torch.bfloat16)
+    wu = (0.2 * torch.randn(FF, K, generator=_gen(135))).to(torch.bfloat16)
+    bg = torch.randn(FF, generator=_gen(136)).to(torch.bfloat16)
+    bu = torch.randn(FF, generator=_gen(137)).to(torch.bfloat16)
+    fused = torch.empty(2 * FF, K, dtype=torch.bfloat16)
+    fused.view(FF // 16, 2, 16, K)[:, 0] = wg.view(FF // 16, 16, K)
+    fused.view(FF // 16, 2, 16, K)[:, 1] = wu.view(FF // 16, 16, K)
+    both = torch.empty(FF // 16, 2, 16, dtype=torch.bfloat16)
+    both[:, 0], both[:, 1] = bg.view(FF // 16, 16), bu.view(FF // 16, 16)
+    w = fused.to(DEV)
+    if blocked:
+        w = ops.block_weight(w)
+    out = torch.zeros(T, FF, dtype=torch.bfloat16, device=DEV)
+    alpha = 1.702 if limit else 1.0
+    assert ops.gemm_gated_extra(x.to(DEV), w, out, 16, both.view(2 * FF).to(DEV) if bias else None, limit, alpha)
+    g, u = x.double() @ wg.double().T, x.double() @ wu.double().T
+    if bias:
+        g, u = g + bg.double(), u + bu.double()
+    if limit:
+        g, u = g.clamp(max=limit), u.clamp(-limit, limit)
+        ref = g * torch.sigmoid(alpha * g) * (u + 1)
+        assert (g == limit).any() and (u == -limit).any()          # (the clamps are reached)
+    else:
+        ref = plain_silu(g) * u
+    assert _rel(out.cpu().double(), ref) < 5e-3
+    # fewer rows than the epilogue's kernels take, or another type: refused, nothing written
+    few = torch.zeros(4, FF, dtype=torch.bfloat16, device=DEV)
+    assert not ops.gemm_gated_extra(x[:4].to(DEV), w, few, 16, None, limit, alpha)
+    assert float(few.abs().max()) == 0.0
+
+
 def test_gemm_dispatch_and_refusals(ops):
     from llmengine.ops import KernelError
     a, w, ref = _bf16_pair(5, 30, 36, 40)               # K = 36 is no multiple of 8: the plain kernel takes it
