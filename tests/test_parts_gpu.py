@@ -440,7 +440,7 @@ def test_toy_routed_feed_forward_position_encoding_and_arrangement():
 
     register_part("feed_forward", "top1_experts", Top1Experts, replace=True)
     register_part("position", "stretched_rotary", StretchedRotary, replace=True)
-    register_part("block", "parallel", ParallelBlock, replace=True)
+    register_part("block", "toy_parallel", ParallelBlock, replace=True)
 
     @dataclass(frozen=True)
     class ToyConfig:
@@ -453,7 +453,7 @@ def test_toy_routed_feed_forward_position_encoding_and_arrangement():
     def build(c):
         norm = PartChoice("rmsnorm", {"size": H, "eps": EPS})
         att = PartChoice("attention", {"hidden_size": H, "num_heads": NQ, "num_kv_heads": NKV, "head_dim": HD})
-        first = LayerSpec(PartChoice("parallel"), att,
+        first = LayerSpec(PartChoice("toy_parallel"), att,
                           PartChoice("top1_experts", {"hidden_size": H, "expert_size": EF, "num_experts": E}),
                           norm, norm, PartChoice("stretched_rotary", {"rotary_dim": ROT, "theta": THETA,
                                                                       "stretch": STRETCH, "max_position": c.max_pos}))
