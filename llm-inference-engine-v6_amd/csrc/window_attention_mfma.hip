@@ -233,17 +233,249 @@ __global__ __launch_bounds__(256, (DSM <= 2 && NVM <= 4) ? 4 : NVM <= 4 ? 3 : 2)
         if (c < nvt) *reinterpret_cast<f32x4*>(a.part_o + at * a.dv + c * 16 + qd * 4) = acc[c];
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same attention for steps in which a request brings many rows (prompts and their portions): the four wavefronts
+// of a workgroup take tiles next to each other, so they walk nearly the same keys; the workgroup fetches every block
+// of 32 keys once, through registers into LDS (two buffers: the next block travels while this one is used, one barrier
+// a block), as keys [32][dk + 8] and values [dv][32], and each wavefront reads its operands from there just before the
+// product that uses them, which leaves registers for four wavefronts a SIMD. Instances exist for values of up to 64 entries (wider ones
+// measured slower than the kernel above). The workgroup walks
+// the blocks that any of its tiles needs; a wavefront passes over a block behind its own last key, and tests visibility
+// only in blocks that some row of its tile does not see whole. Values behind the workgroup's last key are zeroed as
+// they are staged (their page may hold anything). Results are left as by the kernel above, block by block in the same
+// order.
+template <int NVM, bool EDGE, bool CAP>
+__device__ __forceinline__ void shared_block(const WindowArgs& a, const f32x4 (&sc)[2], const bf16* lds_v, f32x4 (&acc)[NVM], float& m,
+                                             float& l, int nvt, int key0, int r, int qd, int pos, bool valid, float inv_cap) {
+    float p[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        float v = sc[j >> 2][j & 3] * a.scale;
+        if (CAP) v = a.softcap * cap_tanh(v * inv_cap);
+        if (EDGE) {
+            const int key = key0 + qd * 8 + j;
+            const bool seen = valid && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
+            v = seen ? v : -INFINITY;
+        }
+        p[j] = v;
+        mx = fmaxf(mx, v);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = (EDGE && m_new == -INFINITY) ? 0.f : m_new;
+    const bool rescale = __any(m_new != m);
+    const float alpha = rescale ? __expf(m - m_use) : 1.f;
+    m = m_new;
+    float sum = 0.f;
+    bf16x8 ph, pl;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float w = __expf(p[j] - m_use);
+        sum += w;
+        const bf16 hi = static_cast<bf16>(w);
+        ph[j] = hi;
+        pl[j] = static_cast<bf16>(w - static_cast<float>(hi));
+    }
+    l = rescale ? l * alpha + sum : l + sum;
+#pragma unroll
+    for (int c = 0; c < NVM; ++c) {
+        if (c < nvt) {
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(lds_v + (c * 16 + r) * 32 + qd * 8);
+            if (rescale) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[c][e] *= alpha;
+            }
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, ph, acc[c], 0, 0, 0);
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pl, acc[c], 0, 0, 0);
+        }
+    }
+}
+
+template <int DSM, int NVM, bool CAP>
+__global__ __launch_bounds__(256, 4) void window_attention_mfma_shared_kernel(WindowArgs a) {
+    constexpr int DKP = DSM * 32 + 8;                       // a staged key's stride (entries): 16 bytes of padding
+    constexpr int K_ELEMS = 32 * DKP, V_ELEMS = NVM * 16 * 32;
+    constexpr int KL = DSM / 2, VL = NVM / 4;               // 16-byte pieces a thread stages of a block's keys and values
+    __shared__ __align__(16) bf16 lds[2 * (K_ELEMS + V_ELEMS)];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 15, qd = lane >> 4;
+    const int s = blockIdx.y / a.nk, kh = blockIdx.y % a.nk;
+    const int vh = kh / a.maps, map = kh % a.maps;
+    const int row0 = a.q_start[s];
+    const int rows_total = (a.q_start[s + 1] - row0) * a.per_value_head;
+    const int RW = blockIdx.x * 64;                         // the workgroup's first row
+    if (RW >= rows_total) return;                           // (the whole workgroup)
+    const int R0 = RW + wave * 16;
+    const bool active = R0 < rows_total;
+    const bool valid = R0 + r < rows_total;
+    const bool all_valid = R0 + 15 < rows_total;
+    const int R = valid ? R0 + r : rows_total - 1;
+    const int t = row0 + R / a.per_value_head;
+    const int qh = (vh * a.per_value_head + R % a.per_value_head) * a.maps + map;
+    const int pos = a.positions[t];
+    const int first_row = active ? R0 : rows_total - 1;
+    const int pos_min = a.positions[row0 + first_row / a.per_value_head];
+    const int last_row = all_valid ? R0 + 15 : rows_total - 1;
+    const int pos_max = a.positions[row0 + last_row / a.per_value_head];
+    // the workgroup's rows
+    const int wg_pos_min = a.positions[row0 + RW / a.per_value_head];
+    const int wg_last = RW + 63 < rows_total ? RW + 63 : rows_total - 1;
+    const int wg_pos_max = a.positions[row0 + wg_last / a.per_value_head];
+    const int* table = a.block_table + static_cast<size_t>(s) * a.max_blocks;
+    const int ds = (a.dk + 31) >> 5, nvt = a.dv >> 4;
+    const int psh = a.page_shift, pmask = a.page - 1;
+    const float inv_cap = a.softcap > 0.f ? 1.0f / a.softcap : 0.f;
+
+    bf16x8 qf[DSM];
+    {
+        const bf16* qrow = a.q + (static_cast<size_t>(t) * a.nq + qh) * a.dk;
+#pragma unroll
+        for (int c = 0; c < DSM; ++c) {
+            const int d0 = c * 32 + qd * 8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qf[c][e] = static_cast<bf16>(0.f);
+            if (c < ds && d0 < a.dk) qf[c] = *reinterpret_cast<const bf16x8*>(qrow + d0);
+        }
+    }
+
+    // the workgroup's blocks of 32 keys: [0, nb_kept) and [first_blk, last_blk]
+    const int lo_min = (a.window > 0 && wg_pos_min - a.window + 1 > 0) ? wg_pos_min - a.window + 1 : 0;
+    int first_blk = lo_min >> 5;
+    const int last_blk = wg_pos_max >> 5;
+    int nb_kept = 0;
+    if (a.window > 0 && a.keep_first > 0) {
+        const int kept = a.keep_first < lo_min ? a.keep_first : lo_min;
+        const int kb = (kept + 31) >> 5;
+        if (kb >= first_blk) first_blk = 0;
+        else nb_kept = kb;
+    }
+    const int nblk = nb_kept + last_blk - first_blk + 1;
+    const int per = (nblk + a.nsplit - 1) / a.nsplit;
+    const int b_begin = blockIdx.z * per;
+    const int b_end = b_begin + per < nblk ? b_begin + per : nblk;
+
+    // staging: piece i of a block's keys is entries 8 (i % cpk) .. of key i / cpk; piece i of its values the keys
+    // 8 (i % 4) .. of value entry i / 4
+    const int cpk = a.dk >> 3;
+    bf16x8 k_st[KL], v_st[VL];
+    auto fetch = [&](int b) {
+        const int key0 = (b < nb_kept ? b : first_blk + b - nb_kept) << 5;
+#pragma unroll
+        for (int i = 0; i < KL; ++i) {
+            const int piece = tid + i * 256;
+            if (piece < 32 * cpk) {
+                int key = key0 + piece / cpk;
+                key = key < wg_pos_max ? key : wg_pos_max;     // (keys behind the workgroup's last are masked by every row)
+                int pg = table[key >> psh];
+                pg = pg < 0 ? 0 : pg;       // (a page that the window has left behind and given back: its keys are masked)
+                k_st[i] = *reinterpret_cast<const bf16x8*>(
+                    a.k_cache + (((static_cast<size_t>(pg) * a.nk + kh) << psh) + (key & pmask)) * a.dk + (piece % cpk) * 8);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VL; ++i) {
+            const int piece = tid + i * 256;
+            if (piece < a.dv * 4) {
+                const int kq = key0 + (piece & 3) * 8;
+                const int kc = kq <= wg_pos_max ? kq : (wg_pos_max & ~7);
+                int pg = table[kc >> psh];
+                pg = pg < 0 ? 0 : pg;
+                bf16x8 v = *reinterpret_cast<const bf16x8*>(
+                    a.v_cache + (((static_cast<size_t>(pg) * a.nv + vh) * a.dv + (piece >> 2)) << psh) + (kc & pmask));
+                if (kq + 7 > wg_pos_max) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (kq + j > wg_pos_max) v[j] = static_cast<bf16>(0.f);
+                }
+                v_st[i] = v;
+            }
+        }
+    };
+    auto stage = [&](int buf) {
+        bf16* lk = lds + buf * (K_ELEMS + V_ELEMS);
+        bf16* lv = lk + K_ELEMS;
+#pragma unroll
+        for (int i = 0; i < KL; ++i) {
+            const int piece = tid + i * 256;
+            if (piece < 32 * cpk) *reinterpret_cast<bf16x8*>(lk + (piece / cpk) * DKP + (piece % cpk) * 8) = k_st[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VL; ++i) {
+            const int piece = tid + i * 256;
+            if (piece < a.dv * 4) *reinterpret_cast<bf16x8*>(lv + (piece >> 2) * 32 + (piece & 3) * 8) = v_st[i];
+        }
+    };
+
+    float m = -INFINITY, l = 0.f;
+    f32x4 acc[NVM];
+#pragma unroll
+    for (int c = 0; c < NVM; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int k_in_block = 8 * (r >> 2) + (r & 3);          // (rows of a 16-key half, as in the kernel above)
+
+    if (b_begin < b_end) {
+        fetch(b_begin);
+        stage(0);
+    }
+    __syncthreads();
+    for (int b = b_begin; b < b_end; ++b) {
+        const int buf = (b - b_begin) & 1;
+        if (b + 1 < b_end) fetch(b + 1);
+        const int key0 = (b < nb_kept ? b : first_blk + b - nb_kept) << 5;
+        // (a block behind this tile's last key, or in front of the window's start of its first row and not among the
+        // kept ones, has no key for it)
+        const bool mine = active && key0 <= pos_max
+                          && (a.window <= 0 || b < nb_kept || key0 + 31 >= pos_min - a.window + 1 || key0 < a.keep_first);
+        if (mine) {
+            const bf16* lk = lds + buf * (K_ELEMS + V_ELEMS);
+            f32x4 sc[2];
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                sc[sub] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < DSM; ++c) {
+                    const int d0 = c * 32 + qd * 8;
+                    if (c < ds) {
+                        bf16x8 kf;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) kf[e] = static_cast<bf16>(0.f);
+                        if (d0 < a.dk) kf = *reinterpret_cast<const bf16x8*>(lk + (k_in_block + 4 * sub) * DKP + d0);
+                        sc[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], sc[sub], 0, 0, 0);
+                    }
+                }
+            }
+            const bool inner = all_valid && b >= nb_kept && key0 + 31 <= pos_min && (a.window <= 0 || pos_max - key0 < a.window);
+            if (inner) shared_block<NVM, false, CAP>(a, sc, lk + K_ELEMS, acc, m, l, nvt, key0, r, qd, pos, valid, inv_cap);
+            else shared_block<NVM, true, CAP>(a, sc, lk + K_ELEMS, acc, m, l, nvt, key0, r, qd, pos, valid, inv_cap);
+        }
+        if (b + 1 < b_end) stage(buf ^ 1);
+        __syncthreads();
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!valid) return;
+    const size_t at = (static_cast<size_t>(blockIdx.z) * a.T + t) * a.nq + qh;
+    if (qd == 0) {
+        a.part_ml[at * 2] = m;
+        a.part_ml[at * 2 + 1] = l;
+    }
+#pragma unroll
+    for (int c = 0; c < NVM; ++c)
+        if (c < nvt) *reinterpret_cast<f32x4*>(a.part_o + at * a.dv + c * 16 + qd * 4) = acc[c];
+}
+
 }  // namespace llme
 
 using namespace llme;
 
-// max_new: the most tokens a request brings to the step (sizes the grid). Refuses (10002) what the kernel does not
+// max_new: the most tokens a request brings to the step (sizes the grid). staged: 0 keeps every step on the kernel without LDS. Refuses (10002) what the kernel does not
 // take: key entries no multiple of 8 or beyond 128, value entries no multiple of 16 or beyond 128, pages that are no
 // power of two from 16 on.
 extern "C" int llme_window_attention_mfma(const void* q, const void* k_cache, const void* v_cache, float* part_o, float* part_ml,
                                           const int* positions, const int* q_start, const int* block_table, int max_blocks, int T,
                                           int S, int max_new, int nq, int nk, int nv, int dk, int dv, int page, float scale,
-                                          float softcap, int window, int keep_first, int nsplit, hipStream_t stream) {
+                                          float softcap, int window, int keep_first, int nsplit, int staged, hipStream_t stream) {
     if (T <= 0 || S <= 0) return 0;
     if (nv <= 0 || nk % nv != 0 || nq % nk != 0 || max_new <= 0 || nsplit <= 0 || window < 0 || keep_first < 0) return kErrBadArgument;
     if (dk % 8 != 0 || dk > 128 || dv % 16 != 0 || dv > 128 || page % 16 != 0 || (page & (page - 1)) != 0) return kErrUnsupported;
@@ -279,11 +511,24 @@ extern "C" int llme_window_attention_mfma(const void* q, const void* k_cache, co
         if (softcap > 0.f) hipLaunchKernelGGL((window_attention_mfma_kernel<DSM, NVM, true>), grid, dim3(256), 0, stream, a); \
         else hipLaunchKernelGGL((window_attention_mfma_kernel<DSM, NVM, false>), grid, dim3(256), 0, stream, a);  \
     } while (0)
-    if (dk <= 64 && dv <= 64) LLME_WMFMA(2, 4);
+#define LLME_WSHARED(DSM, NVM)                                                                                          \
+    do {                                                                                                                \
+        if (softcap > 0.f) hipLaunchKernelGGL((window_attention_mfma_shared_kernel<DSM, NVM, true>), grid, dim3(256), 0, stream, a); \
+        else hipLaunchKernelGGL((window_attention_mfma_shared_kernel<DSM, NVM, false>), grid, dim3(256), 0, stream, a);  \
+    } while (0)
+    // a request that brings a workgroup's 64 rows or more, values of up to 64 entries: the blocks staged once a workgroup;
+    // fewer rows (decoded tokens, short portions): a wavefront on its own
+    // (with values beyond 64 entries the staged kernel measured slower: 170 against 156 us over a prompt of 2,048)
+    const bool shared = staged != 0 && static_cast<long>(max_new) * a.per_value_head >= 64 && dv <= 64;
+    if (shared) {
+        if (dk <= 64) LLME_WSHARED(2, 4);
+        else LLME_WSHARED(4, 4);
+    } else if (dk <= 64 && dv <= 64) LLME_WMFMA(2, 4);
     else if (dk <= 64) LLME_WMFMA(2, 8);
     else if (dv <= 64) LLME_WMFMA(4, 4);
     else LLME_WMFMA(4, 8);
 #undef LLME_WMFMA
+#undef LLME_WSHARED
     return launch_status();
 }
 

@@ -69,7 +69,8 @@ def qk_prepare(p: torch.Tensor, step, block_table: torch.Tensor, q_out: torch.Te
 
 
 declare("llme_window_attention_mfma", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
-                                       _i, _vp])
+                                       _i, _i, _vp])
+WINDOW_MFMA_STAGED = True           # prompts' blocks of keys staged once a workgroup through LDS (False: measurements, tests)
 WINDOW_MFMA_MAX_ENTRIES = 128       # entries of a key or value head that the matrix-core kernel holds
 WINDOW_MFMA_MAX_RUNS = 32
 
@@ -114,7 +115,7 @@ def _fast_window_attention(q, k_cache, v_cache, step, block_table, nq, scale, so
     check(entry("llme_window_attention_mfma")(ptr(q), ptr(k_cache), ptr(v_cache), ptr(part_o), ptr(part_ml), ptr(step.positions),
                                               ptr(step.q_start), ptr(block_table), block_table.shape[1], T, step.num_seqs, max_new,
                                               nq, nk, nv, dk, dv, page, float(scale), float(softcap), int(window), int(keep_first),
-                                              runs, stream()), "window_attention_mfma")
+                                              runs, 1 if WINDOW_MFMA_STAGED else 0, stream()), "window_attention_mfma")
     return part_o, part_ml
 
 

@@ -173,6 +173,29 @@ def test_the_matrix_core_attention_at_other_sizes(tmp_path, name):
         assert _mean(got, ref) < 6e-2
 
 
+@pytest.mark.parametrize("name", sorted(MATRIX_CORES))
+def test_staged_blocks_of_keys_give_what_a_wavefront_alone_gives(tmp_path, name):
+    """Prompts' attention with every block of keys staged once a workgroup through LDS walks the same blocks in the same
+    order as the kernel in which a wavefront fetches its own: the logits agree to the last bits, whole and in portions."""
+    from llmengine.ops import window
+    cfg = MATRIX_CORES[name]
+    engine, weights = _engine(tmp_path, cfg, 22, "bf16")
+    V = cfg["vocab"]
+    requests = {"a": _tokens(333, V, 5), "b": _tokens(70, V, 6), "c": _tokens(17, V, 7)}
+    for steps in (replay.whole(requests), replay.portions(requests, sizes=(65, 16, 130, 23)),
+                  replay.mixed(requests, max_live=3, sizes=(90, 40, 2), seed=9)):
+        got = {}
+        for staged in (True, False):
+            window.WINDOW_MFMA_STAGED = staged
+            try:
+                got[staged] = _stacked(replay.run_trace(engine, engine.new_cache(replay.trace_peak_tokens(steps, 16) // 16, 16, 3), steps))
+            finally:
+                window.WINDOW_MFMA_STAGED = True
+        for rid in requests:
+            scale = float(np.sqrt(np.mean(got[False][rid] ** 2)))
+            assert float(np.abs(got[True][rid] - got[False][rid]).max()) <= 1e-5 * scale
+
+
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 def test_a_batch_of_unequal_requests_against_each_alone(tmp_path, dtype):
     cfg = zm.ALIGNED
