@@ -39,14 +39,12 @@ struct WindowArgs {
     float scale, softcap;
 };
 
-// tanh for the capped scores: the odd series where |y| is small (there 1 - 2 / (e^2y + 1) would cancel), the
-// exponential elsewhere; both in 32-bit with the hardware's exponential and reciprocal.
-__device__ __forceinline__ float cap_tanh(float y) {
-    const float y2 = y * y;
-    const float series = y * (1.f + y2 * (-1.f / 3.f + y2 * (2.f / 15.f)));
-    const float e = __expf(2.f * y);
-    const float wide = 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
-    return fabsf(y) < 0.05f ? series : wide;
+// A capped score from the raw product: cap tanh(scale s / cap) = cap - 2 cap / (e^(2 scale s / cap) + 1), with the
+// hardware's 32-bit power of two and reciprocal; `k` is 2 scale log2(e) / cap. (Where the score is near zero the
+// result is exact to about cap x 1e-7.)
+__device__ __forceinline__ float capped_score(float s, float k, float cap) {
+    const float e = __builtin_amdgcn_exp2f(s * k);
+    return fmaf(-2.f * cap, __builtin_amdgcn_rcpf(e + 1.f), cap);
 }
 
 // One block of 32 keys for a tile: scores in sc (this lane's row, keys key0 + 8 qd + j for j = 4 sub + e), values in vf.
@@ -59,8 +57,8 @@ __device__ __forceinline__ void window_block(const WindowArgs& a, const f32x4 (&
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        float v = sc[j >> 2][j & 3] * a.scale;
-        if (CAP) v = a.softcap * cap_tanh(v * inv_cap);
+        const float v0 = sc[j >> 2][j & 3];
+        float v = CAP ? capped_score(v0, inv_cap, a.softcap) : v0 * a.scale;
         if (EDGE) {
             const int key = key0 + qd * 8 + j;
             const bool seen = valid && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
@@ -132,7 +130,7 @@ __global__ __launch_bounds__(256, (DSM <= 2 && NVM <= 4) ? 4 : NVM <= 4 ? 3 : 2)
     const int* table = a.block_table + static_cast<size_t>(s) * a.max_blocks;
     const int ds = (a.dk + 31) >> 5, nvt = a.dv >> 4;
     const int psh = a.page_shift, pmask = a.page - 1;
-    const float inv_cap = a.softcap > 0.f ? 1.0f / a.softcap : 0.f;
+    const float inv_cap = a.softcap > 0.f ? 2.0f * 1.4426950408889634f * a.scale / a.softcap : 0.f;     // (capped_score's k)
 
     bf16x8 qf[DSM];
     {
@@ -251,8 +249,8 @@ __device__ __forceinline__ void shared_block(const WindowArgs& a, const f32x4 (&
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        float v = sc[j >> 2][j & 3] * a.scale;
-        if (CAP) v = a.softcap * cap_tanh(v * inv_cap);
+        const float v0 = sc[j >> 2][j & 3];
+        float v = CAP ? capped_score(v0, inv_cap, a.softcap) : v0 * a.scale;
         if (EDGE) {
             const int key = key0 + qd * 8 + j;
             const bool seen = valid && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
@@ -326,7 +324,7 @@ __global__ __launch_bounds__(256, 4) void window_attention_mfma_shared_kernel(Wi
     const int* table = a.block_table + static_cast<size_t>(s) * a.max_blocks;
     const int ds = (a.dk + 31) >> 5, nvt = a.dv >> 4;
     const int psh = a.page_shift, pmask = a.page - 1;
-    const float inv_cap = a.softcap > 0.f ? 1.0f / a.softcap : 0.f;
+    const float inv_cap = a.softcap > 0.f ? 2.0f * 1.4426950408889634f * a.scale / a.softcap : 0.f;     // (capped_score's k)
 
     bf16x8 qf[DSM];
     {
