@@ -4,6 +4,8 @@
 //     alternating groups (biases in the same order, or none), with the activations
 //       0 silu, 1 rectifier, 2 gelu (tanh form),
 //       3 clamped swish: g = min(gate, limit), u = clamp(up, -limit, limit), out = g * sigmoid(alpha g) * (u + 1);
+//     with `row_pair` and `pair_scale` the sums of row t are first multiplied by pair_scale[row_pair[t]] (0 where the row
+//     holds no pair): an expert that runs on its weight times the input, the weight taken out of the two products;
 //   * add_row_bias: every row of a 32-bit matrix gets the same row added (the bias of an output product that
 //     accumulates into the residual stream);
 //   * table_route: a token's experts read from a table by its id, each weighing 1 / top;
@@ -15,7 +17,8 @@ namespace llme {
 
 template <typename TB, typename TO>
 __global__ void gated_bias_act_kernel(const float* __restrict__ gu, int ld, const TB* __restrict__ bias, TO* __restrict__ out, int FF,
-                                      int group, size_t total, int act, float limit, float alpha) {
+                                      int group, size_t total, int act, float limit, float alpha,
+                                      const int* __restrict__ row_pair, const float* __restrict__ pair_scale) {
     const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const size_t t = idx / FF;
@@ -23,6 +26,12 @@ __global__ void gated_bias_act_kernel(const float* __restrict__ gu, int ld, cons
     const int col = (j / group) * 2 * group + (j % group);
     float g = gu[t * ld + col];
     float u = gu[t * ld + col + group];
+    if (row_pair != nullptr) {
+        const int pair = row_pair[t];
+        const float sc = pair < 0 ? 0.f : pair_scale[pair];
+        g *= sc;
+        u *= sc;
+    }
     if (bias != nullptr) {
         g += to_float(bias[col]);
         u += to_float(bias[col + group]);
@@ -71,14 +80,16 @@ __global__ void concat_rows_kernel(const float* __restrict__ a, const float* __r
 using namespace llme;
 
 extern "C" int llme_gated_bias_act(const float* gu, int ld, const void* bias, int bias_dtype, void* out, int out_dtype, int T, int FF,
-                                   int group, int act, float limit, float alpha, hipStream_t stream) {
+                                   int group, int act, float limit, float alpha, const int* row_pair, const float* pair_scale,
+                                   hipStream_t stream) {
     if (T <= 0) return 0;
     if (group <= 0 || FF % group != 0 || act < 0 || act > 3 || ld < 2 * FF) return kErrBadArgument;
+    if ((row_pair == nullptr) != (pair_scale == nullptr)) return kErrBadArgument;
     const size_t total = static_cast<size_t>(T) * FF;
     const dim3 grid(static_cast<unsigned>((total + 255) / 256));
 #define LLME_GBA(TB, TO)                                                                                              \
     hipLaunchKernelGGL((gated_bias_act_kernel<TB, TO>), grid, dim3(256), 0, stream, gu, ld, static_cast<const TB*>(bias), \
-                       static_cast<TO*>(out), FF, group, total, act, limit, alpha)
+                       static_cast<TO*>(out), FF, group, total, act, limit, alpha, row_pair, pair_scale)
     const bool bb = bias != nullptr && bias_dtype == kBF16;
     if (out_dtype == kF32 && !bb) LLME_GBA(float, float);
     else if (out_dtype == kF32 && bb) LLME_GBA(bf16, float);

@@ -1,8 +1,8 @@
 // Mixture of experts: every token runs `top` of E small gated feed-forward layers.
 //
-//   moe_route    logits [T, E] (32-bit) -> per token the `top` experts with the largest softmax scores
-//                (the lower index wins a tie) and their weights = score * scale, renormalised over the
-//                chosen ones or not; pairs are numbered t * top + k
+//   moe_route    logits [T, E] (32-bit) -> per token the `top` experts with the largest scores (softmax over
+//                the experts, or a sigmoid of each logit on its own; the lower index wins a tie) and their
+//                weights = score * scale, renormalised over the chosen ones or not; pairs are numbered t * top + k
 //   moe_plan     the pairs grouped by expert: every expert's pairs take a run of places padded to whole
 //                tiles of `tile` rows; place -> pair (-1: padding), pair -> place, tile -> expert, number
 //                of tiles. One workgroup; which place of its expert's run a pair takes depends on the
@@ -10,7 +10,7 @@
 //   moe_gemm     per tile of places: rows gathered (token = pair / top, or the place itself) times the
 //                tile's expert's matrix [N, K]; plain or gated (act(gate) * up, gate and up rows in one matrix);
 //                the plain-precision kernel; bfloat16 steps take the grouped instances of the matrix-core tile kernel
-//   moe_combine  out[t] (+)= sum_k weight[t, k] * y[place of (t, k)], k in order
+//   moe_combine  out[t] (+)= sum_k weight[t, k] * y[place of (t, k)], k in order (no weights: each counts once)
 //
 // Everything that depends on the routing is read from device memory: a step's launches are the same
 // whatever the tokens choose (grids are sized for the most tiles there can be; workgroups beyond the
@@ -29,7 +29,7 @@ __device__ __forceinline__ float moe_act(float g, int act) {
 constexpr int kMoeMaxPerLane = 16;      // experts per lane: up to 1024 experts
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int T, int E, int top,
-                                                        float scale, int renorm, int* __restrict__ ids,
+                                                        float scale, int renorm, int sigmoid, int* __restrict__ ids,
                                                         float* __restrict__ wts) {
     const int lane = threadIdx.x & (kWave - 1);
     const int t = blockIdx.x * 4 + threadIdx.x / kWave;
@@ -47,10 +47,10 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < kMoeMaxPerLane; ++i) {
-        v[i] = expf(v[i] - mx);                 // 0 beyond E
+        v[i] = sigmoid ? 1.0f / (1.0f + expf(-v[i])) : expf(v[i] - mx);                 // 0 beyond E
         sum += v[i];
     }
-    const float inv = 1.0f / wave_sum(sum);
+    const float inv = sigmoid ? 1.0f : 1.0f / wave_sum(sum);
     float chosen_sum = 0.f;
     for (int k = 0; k < top; ++k) {
         float best = -1.f;
@@ -195,7 +195,7 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, const int* __res
     const int c = static_cast<int>(idx % H);
     float s = accumulate ? out[idx] : 0.f;
     for (int k = 0; k < top; ++k)
-        s = fmaf(wts[t * top + k], y[static_cast<size_t>(pair_place[t * top + k]) * H + c], s);
+        s = fmaf(wts != nullptr ? wts[t * top + k] : 1.0f, y[static_cast<size_t>(pair_place[t * top + k]) * H + c], s);
     out[idx] = s;
 }
 
@@ -203,12 +203,12 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, const int* __res
 
 using namespace llme;
 
-extern "C" int llme_moe_route(const float* logits, int T, int E, int top, float scale, int renorm, int* ids, float* wts,
-                              hipStream_t stream) {
+extern "C" int llme_moe_route(const float* logits, int T, int E, int top, float scale, int renorm, int sigmoid, int* ids,
+                              float* wts, hipStream_t stream) {
     if (T <= 0) return 0;
     if (E <= 0 || top <= 0 || top > E) return kErrBadArgument;
     if (E > kMoeMaxPerLane * kWave) return kErrUnsupported;
-    hipLaunchKernelGGL(moe_route_kernel, dim3((T + 3) / 4), dim3(256), 0, stream, logits, T, E, top, scale, renorm, ids, wts);
+    hipLaunchKernelGGL(moe_route_kernel, dim3((T + 3) / 4), dim3(256), 0, stream, logits, T, E, top, scale, renorm, sigmoid, ids, wts);
     return launch_status();
 }
 

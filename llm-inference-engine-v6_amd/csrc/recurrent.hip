@@ -306,6 +306,18 @@ __global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restric
     decay[static_cast<size_t>(t) * n_dec + e] = expf(-expf(A_log[h]) * softplusf_(z));
 }
 
+// decay[t, e] = sigmoid(z[t, e] + bias[e])^(1 / tau) = exp(-softplus(-(z + bias)) / tau): a decay per channel from a
+// logit, flattened by a temperature. z is a column range of a 32-bit buffer; bias (null: none) in its stored type.
+template <typename TW>
+__global__ __launch_bounds__(256) void sigmoid_decay_kernel(const float* __restrict__ z, int ld, const TW* __restrict__ bias,
+                                                            float inv_tau, float* __restrict__ decay, int n) {
+    const int t = blockIdx.y;
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= n) return;
+    const float x = z[static_cast<size_t>(t) * ld + e] + (bias != nullptr ? to_float(bias[e]) : 0.f);
+    decay[static_cast<size_t>(t) * n + e] = expf(-softplusf_(-x) * inv_tau);
+}
+
 // The delta rule. State M per request and head (32-bit, in the request's slot), kept as [vdim][dim]: a column's key
 // channels lie together. Per token:
 //   M <- g * M (g per key channel or one per head);  w = beta (v - M^T k);  M <- M + k w^T;  o = M^T q.
@@ -329,12 +341,15 @@ __device__ __forceinline__ float sum_of_lanes(float v) {
     return v;
 }
 
-template <int R, int LPC, bool PER_CHANNEL>
+// DELTA false is the plain linear rule (gated linear attention): nothing is read back before the write,
+//   M <- g * M;  M <- M + k v^T;  o = M^T q,
+// and beta is not looked at. Every read is multiplied by o_scale (a scale on the queries).
+template <int R, int LPC, bool PER_CHANNEL, bool DELTA>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ qkv, int ld, int q_col, int k_col, int v_col,
                                                          const float* __restrict__ beta, const float* __restrict__ decay,
                                                          float* __restrict__ state, const int* __restrict__ q_start,
-                                                         const int* __restrict__ slots, float* __restrict__ o, int heads,
-                                                         int kv_heads, int dim, int vdim) {
+ const int* __restrict__ slots, float* __restrict__ o, int heads,
+                                                         int kv_heads, int dim, int vdim, float o_scale) {
     constexpr int DP = LPC * R;                             // a row's k (q, decay) padded with zeros to this many
     constexpr int kDeltaCols = 256 / LPC;                   // columns of the state a workgroup owns
     constexpr int NV = PER_CHANNEL ? 3 : 2;
@@ -383,7 +398,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
                 const int y = x - NV * DP;
                 if (y < kDeltaCols) {
                     if (col0 + y < vdim) { src[i] = qkv + t * ld + v_col + h * vdim + col0 + y; advance[i] = kDeltaRows * ld; }
-                } else if (y == kDeltaCols) {
+                } else if (y == kDeltaCols && DELTA) {
                     src[i] = beta + t * heads + h;
                     advance[i] = kDeltaRows * heads;
                 } else if (y == kDeltaCols + 1 && !PER_CHANNEL) {
@@ -453,8 +468,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
                 m[i] *= PER_CHANNEL ? gg[i] : g_head;
                 dots[i % 2] += m[i] * kk[i];
             }
-            const float dot = sum_of_lanes<LPC>(dots[0] + dots[1]);
-            const float w = bt * (vv - dot);
+            const float w = DELTA ? bt * (vv - sum_of_lanes<LPC>(dots[0] + dots[1])) : vv;
             float reads[2] = {0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < R; ++i) {
@@ -462,7 +476,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
                 reads[i % 2] += m[i] * qq[i];
             }
             const float read = sum_of_lanes<LPC>(reads[0] + reads[1]);
-            if (live && l == 0) o[static_cast<size_t>(t0 + tt) * heads * vdim + h * vdim + col] = read;
+            if (live && l == 0) o[static_cast<size_t>(t0 + tt) * heads * vdim + h * vdim + col] = read * o_scale;
         };
         if (nt == kDeltaRows) {             // a whole block: no test between its rows, so that the rows' loads from LDS run ahead
 #pragma unroll
@@ -650,24 +664,40 @@ extern "C" int llme_delta_gates(const void* b_in, int ld_b, const void* a_in, in
     return launch_status();
 }
 
+extern "C" int llme_sigmoid_decay(const void* z, int ld, const void* bias, int w_dtype, float tau, void* decay, int T, int n,
+                                  hipStream_t stream) {
+    if (T <= 0 || n <= 0) return 0;
+    if (!(tau > 0.f) || ld < n) return kErrBadArgument;
+    const dim3 grid((n + 255) / 256, T);
+    LLME_BY_W(w_dtype, (sigmoid_decay_kernel<TW><<<grid, 256, 0, stream>>>(static_cast<const float*>(z), ld, static_cast<const TW*>(bias),
+                                                                       1.0f / tau, static_cast<float*>(decay), n)));
+    return launch_status();
+}
+
 template <int R, int LPC>
 static void launch_delta_rule(bool per_channel, int n_seq, hipStream_t stream, const float* qkv, int ld, int q_col, int k_col,
                               int v_col, const float* beta, const float* decay, float* state, const int* q_start,
-                              const int* slots, float* o, int heads, int kv_heads, int dim, int vdim) {
+                              const int* slots, float* o, int heads, int kv_heads, int dim, int vdim, float o_scale) {
     const dim3 grid((vdim + 256 / LPC - 1) / (256 / LPC), heads, n_seq);
-    if (per_channel)
-        delta_rule_kernel<R, LPC, true><<<grid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots, o,
-                                                             heads, kv_heads, dim, vdim);
-    else
-        delta_rule_kernel<R, LPC, false><<<grid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots, o,
-                                                              heads, kv_heads, dim, vdim);
+#define LLME_DR(PC, DL)                                                                                                          \
+    delta_rule_kernel<R, LPC, PC, DL><<<grid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots, o, \
+                                                                 heads, kv_heads, dim, vdim, o_scale)
+    if (beta != nullptr) {
+        if (per_channel) LLME_DR(true, true);
+        else LLME_DR(false, true);
+    } else {
+        if (per_channel) LLME_DR(true, false);
+        else LLME_DR(false, false);
+    }
+#undef LLME_DR
 }
 
 // qkv [T, ld] 32-bit with unit q at q_col, unit k at k_col (kv_heads x dim each) and v at v_col (heads x vdim);
-// beta [T, heads]; decay [T, heads, dim] or [T, heads]; state [slots, heads, vdim, dim]; o [T, heads, vdim] 32-bit.
+// beta [T, heads], or null for the linear rule; decay [T, heads, dim] or [T, heads]; state [slots, heads, vdim, dim];
+// o [T, heads, vdim] 32-bit, times o_scale.
 extern "C" int llme_delta_rule(const void* qkv, int ld, int q_col, int k_col, int v_col, const void* beta, const void* decay,
                                int per_channel, void* state, const void* q_start, const void* slots, void* o, int n_seq,
-                               int heads, int kv_heads, int dim, int vdim, hipStream_t stream) {
+                               int heads, int kv_heads, int dim, int vdim, float o_scale, hipStream_t stream) {
     if (n_seq <= 0 || heads <= 0) return 0;
     if (kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return kErrBadArgument;
     if (dim > 256) return kErrUnsupported;
@@ -675,7 +705,7 @@ extern "C" int llme_delta_rule(const void* qkv, int ld, int q_col, int k_col, in
     launch_delta_rule<R_, L_>(per_channel != 0, n_seq, stream, static_cast<const float*>(qkv), ld, q_col, k_col, v_col, \
                           static_cast<const float*>(beta), static_cast<const float*>(decay), static_cast<float*>(state), \
                           static_cast<const int*>(q_start), static_cast<const int*>(slots), static_cast<float*>(o), heads, \
-                          kv_heads, dim, vdim)
+                          kv_heads, dim, vdim, o_scale)
     if (dim <= 16) LLME_DELTA(2, 8);
     else if (dim <= 32) LLME_DELTA(4, 8);
     else if (dim <= 64) LLME_DELTA(4, 16);

@@ -2,6 +2,8 @@
 //   h[t] += w_post * y[t] / sqrt(mean(y[t]^2) + eps)
 // and, in the same pass over the row, the norm in front of the next sublayer:
 //   x[t] = w_next * h[t] / sqrt(mean(h[t]^2) + eps)      (h as just updated)
+// or, where x is asked for without a weight, the updated row as it is in the activation type (x[t] = h[t]: layers
+// whose sublayers read the stream itself and are normed behind).
 // y and h are 32-bit; the weights multiply as given (a norm whose checkpoint stores the distance from one
 // hands over 1 + w). The products are evaluated (w * v) * inv, as the norm kernel evaluates them, so that a
 // row is rounded to the same values whichever kernel norms it. One workgroup a row; the row waits in LDS
@@ -33,9 +35,13 @@ __global__ __launch_bounds__(256) void norm_add_kernel(const float* __restrict__
         row[i] = v;
         ss2 = fmaf(v, v, ss2);
     }
-    if (w_next == nullptr) return;
-    const float inv2 = 1.0f / sqrtf(block_sum(ss2, scratch, 4) / static_cast<float>(H) + eps);
+    if (x_out == nullptr) return;
     TO* xr = x_out + static_cast<size_t>(t) * H;
+    if (w_next == nullptr) {
+        for (int i = threadIdx.x; i < H; i += 256) xr[i] = from_float<TO>(row[i]);
+        return;
+    }
+    const float inv2 = 1.0f / sqrtf(block_sum(ss2, scratch, 4) / static_cast<float>(H) + eps);
     for (int i = threadIdx.x; i < H; i += 256) xr[i] = from_float<TO>((to_float(w_next[i]) * row[i]) * inv2);
 }
 
@@ -102,9 +108,17 @@ __global__ __launch_bounds__(256) void norm_add_vec_kernel(const float* __restri
         }
         if (i < H) na_store4(hr + i, hv[k]);
     }
-    if (w_next == nullptr) return;
-    const float inv2 = 1.0f / sqrtf(block_sum(ss2, scratch, 4) / static_cast<float>(H) + eps);
+    if (x_out == nullptr) return;
     TO* xr = x_out + static_cast<size_t>(t) * H;
+    if (w_next == nullptr) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int i = (threadIdx.x + 256 * k) * 4;
+            if (i < H) na_store4(xr + i, hv[k]);
+        }
+        return;
+    }
+    const float inv2 = 1.0f / sqrtf(block_sum(ss2, scratch, 4) / static_cast<float>(H) + eps);
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
         const int i = (threadIdx.x + 256 * k) * 4;
@@ -147,8 +161,13 @@ extern "C" int llme_norm_add(const float* y, const void* w_post, int w_dtype, fl
                                static_cast<TO*>(x_out), H, eps);                                          \
     } while (0)
     if (w_next == nullptr) {
-        if (w_dtype == kF32) LLME_NA(float, float, float);
-        else if (w_dtype == kBF16) LLME_NA(bf16, float, float);
+        // nothing more, or the updated rows as they are in x_out's type
+        const bool xb = x_out != nullptr && xo_dtype == kBF16;
+        if (x_out != nullptr && xo_dtype != kBF16 && xo_dtype != kF32) return kErrBadArgument;
+        if (w_dtype == kF32 && !xb) LLME_NA(float, float, float);
+        else if (w_dtype == kF32 && xb) LLME_NA(float, float, bf16);
+        else if (w_dtype == kBF16 && !xb) LLME_NA(bf16, float, float);
+        else if (w_dtype == kBF16 && xb) LLME_NA(bf16, float, bf16);
         else return kErrBadArgument;
         return launch_status();
     }

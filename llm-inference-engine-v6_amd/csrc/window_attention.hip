@@ -5,14 +5,19 @@
 //     qh = (head, map) reads key head (head / (heads / nv)) * maps + map and value head head / (heads / nv);
 //   * a score is scale * q . k, then softcap * tanh(score / softcap) where softcap > 0;
 //   * a query at position p sees key j <= p with p - j < window (window 0: every j <= p) or j < keep_first (the first
-//     tokens of a sequence stay visible behind a sliding window, at their true positions).
+//     tokens of a sequence stay visible behind a sliding window, at their true positions);
+//   * `slopes` (one number a head): a score loses slope_h (p - j), a bias that grows with the distance;
+//   * `sinks` (one number a head): the softmax's denominator also holds e^(sink_h), a key without a value.
 //
 // Three steps: `qk_prepare` turns the input product's 32-bit rows into queries and cache entries (an RMS norm per
 // head with a weight over the head's entries where given, a rotation of the first `rot` entries by position x
-// frequency), an attention kernel leaves per run of keys the maximum, the sum and the unscaled weighted values of
+// frequency, entry i with entry i + rot / 2 or, `pairs` = 1, entry 2 i with entry 2 i + 1; queries times a temperature
+// 1 + coef ln(floor((p + 1) / every) + 1) where `every` > 0; nk = 0: the layer reads another layer's keys and values
+// and only its queries are made), an attention kernel leaves per run of keys the maximum, the sum and the unscaled weighted values of
 // every (token, query head), and `window_attention_finish` joins the runs in a fixed order and applies what a mixer
-// does to a head's result before its output product: nothing, an element-wise sigmoid gate, or the difference of a
-// head's two maps, o = a_1 - lambda a_2, divided by its root mean square and scaled.
+// does to a head's result before its output product: nothing, an element-wise sigmoid gate, a sigmoid gate of one
+// number a head, or the difference of a head's two maps, o = a_1 - lambda a_2, divided by its root mean square; all
+// times a constant.
 //
 // Scores, weights, norms, angles and sums over keys are 32-bit; q, k and v are read in their storage type.
 // The kernel in this file is the plain-precision one (any sizes, both types); the matrix-core one is in
@@ -35,7 +40,8 @@ constexpr int kMaxHeadEntries = 256;
 template <typename TQ, typename TC, typename TW>
 __global__ __launch_bounds__(256) void qk_prepare_kernel(const float* __restrict__ p, int ld, int nq, int nk, int nv, int dk, int dv,
                                                          int k_col, int v_col, const TW* __restrict__ wq, const TW* __restrict__ wk,
-                                                         float eps, const float* __restrict__ inv_freq, int rot,
+                                                         float eps, const float* __restrict__ inv_freq, int rot, int pairs,
+                                                         float qt_coef, int qt_every,
                                                          const int* __restrict__ positions, const int* __restrict__ seq_idx,
                                                          const int* __restrict__ block_table, int max_blocks,
                                                          TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
@@ -46,9 +52,11 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(const float* __restrict
     const int pos = positions[t];
     const float fpos = static_cast<float>(pos);
     const float* row = p + static_cast<size_t>(t) * ld;
-    const int pg = block_table[static_cast<size_t>(seq_idx[t]) * max_blocks + pos / page];
+    const int pg = nk > 0 ? block_table[static_cast<size_t>(seq_idx[t]) * max_blocks + pos / page] : 0;
     const int in_page = pos % page;
     const int half = rot / 2;
+    // the queries' temperature at this position (32-bit)
+    const float q_temp = qt_every > 0 ? 1.0f + qt_coef * logf(static_cast<float>((pos + 1) / qt_every + 1)) : 1.0f;
     for (int f = threadIdx.x; f < half; f += 256) {
         float sn, cs;
         sincosf(fpos * inv_freq[f], &sn, &cs);
@@ -71,21 +79,22 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(const float* __restrict
             const float raw = hp[e];
             float v = w != nullptr ? raw * r * to_float(w[e]) : raw;
             if (e < rot) {
-                const int f = e < half ? e : e - half;
-                const int pe = e < half ? e + half : e - half;
+                const bool first = pairs ? (e & 1) == 0 : e < half;
+                const int f = pairs ? e >> 1 : (e < half ? e : e - half);
+                const int pe = pairs ? e ^ 1 : (e < half ? e + half : e - half);
                 const float other = w != nullptr ? hp[pe] * r * to_float(w[pe]) : hp[pe];
                 const float sn = sn_t[f], cs = cs_t[f];
-                v = e < half ? v * cs - other * sn : v * cs + other * sn;
+                v = first ? v * cs - other * sn : v * cs + other * sn;
             }
             if (is_q) {
-                q_out[(static_cast<size_t>(t) * nq + head) * dk + e] = from_float<TQ>(v);
+                q_out[(static_cast<size_t>(t) * nq + head) * dk + e] = from_float<TQ>(v * q_temp);
             } else {
                 k_cache[((static_cast<size_t>(pg) * nk + head) * page + in_page) * dk + e] = from_float<TC>(v);
                 if (v_col < 0) v_cache[((static_cast<size_t>(pg) * nv + head) * dv + e) * page + in_page] = from_float<TC>(raw);
             }
         }
     }
-    if (v_col >= 0) {
+    if (v_col >= 0 && nv > 0) {
         const float* vp = row + v_col;
         for (int e = blockIdx.y * 256 + threadIdx.x; e < nv * dv; e += 256 * gridDim.y)
             v_cache[((static_cast<size_t>(pg) * nv + e / dv) * dv + e % dv) * page + in_page] = from_float<TC>(vp[e]);
@@ -102,7 +111,7 @@ __global__ __launch_bounds__(NW * 64) void window_attention_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache, float* __restrict__ part_o,
     float* __restrict__ part_ml, const int* __restrict__ positions, const int* __restrict__ seq_idx,
     const int* __restrict__ block_table, int max_blocks, int nq, int nk, int nv, int maps, int dk, int dv, int page, float scale,
-    float softcap, int window, int keep_first) {
+    float softcap, int window, int keep_first, const float* __restrict__ slopes) {
     constexpr int PER_LANE = kMaxHeadEntries / kWave;
     __shared__ float qs[kMaxHeadEntries];
     __shared__ float join_m[NW], join_l[NW];
@@ -117,6 +126,7 @@ __global__ __launch_bounds__(NW * 64) void window_attention_kernel(
     const int hi = pos + 1;
     const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
     const int kept = keep_first < lo ? keep_first : lo;        // the first tokens that lie in front of the window
+    const float slope = slopes != nullptr ? slopes[head] : 0.f;
 
     const TQ* qrow = q + (static_cast<size_t>(t) * nq + qh) * dk;
     for (int d = threadIdx.x; d < dk; d += NW * kWave) qs[d] = to_float(qrow[d]);
@@ -137,6 +147,7 @@ __global__ __launch_bounds__(NW * 64) void window_attention_kernel(
                 for (int d = 0; d < dk; ++d) dot = fmaf(qs[d], to_float(kr[d]), dot);
                 sc = dot * scale;
                 if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
+                sc -= slope * static_cast<float>(pos - key);
             }
             const float m_new = fmaxf(m, wave_max(sc));
             const float alpha = expf(m - m_new);
@@ -193,16 +204,18 @@ __global__ __launch_bounds__(NW * 64) void window_attention_kernel(
     }
 }
 
-enum FinishMode : int { kFinishPlain = 0, kFinishGate = 1, kFinishDifference = 2 };
+enum FinishMode : int { kFinishPlain = 0, kFinishGate = 1, kFinishDifference = 2, kFinishHeadGate = 3 };
 
 // One wavefront per (token, head): the runs of each of the head's maps joined in the order of the runs, then the
-// mixer's last step. gate [T, ld_gate] 32-bit, one entry per output entry (kFinishGate). kFinishDifference:
-// o = a_1 - lambda a_2 over the head's two maps, o / sqrt(mean(o^2) + eps) * out_scale.
+// mixer's last step. gate [T, ld_gate] 32-bit, one entry per output entry (kFinishGate) or one per head
+// (kFinishHeadGate). kFinishDifference: o = a_1 - lambda a_2 over the head's two maps, o / sqrt(mean(o^2) + eps).
+// sinks [heads] (32-bit, or null; one map a head): the joined sum also holds e^(sink - maximum). All times out_scale.
 template <typename TO, int MODE>
 __global__ __launch_bounds__(256) void window_attention_finish_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                                       int runs, int T, int heads, int maps, int dv,
                                                                       const float* __restrict__ gate, int ld_gate, float lambda,
-                                                                      float eps, float out_scale, TO* __restrict__ out, int ld_out) {
+                                                                      float eps, float out_scale, const float* __restrict__ sinks,
+                                                                      TO* __restrict__ out, int ld_out) {
     constexpr int PER_LANE = kMaxHeadEntries / kWave;
     const int lane = threadIdx.x & 63;
     const size_t item = static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
@@ -276,6 +289,16 @@ __global__ __launch_bounds__(256) void window_attention_finish_kernel(const floa
                 }
         }
     }
+    if (MAPS == 1 && sinks != nullptr) {
+        // the sink joins like a run that holds one weight and no value
+        const float m0 = runs == 1 ? part_ml[at0 * 2] : mx[0];
+        const float sk = sinks[head];
+        const float top = fmaxf(m0, sk);
+        const float f = m0 == -INFINITY ? 0.f : expf(m0 - top);
+        l[0] = fmaf(l[0], f, expf(sk - top));
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) a[0][i] *= f;
+    }
     float o[PER_LANE];
     {
         const float inv = 1.0f / l[0];
@@ -287,13 +310,14 @@ __global__ __launch_bounds__(256) void window_attention_finish_kernel(const floa
             for (int i = 0; i < PER_LANE; ++i) o[i] = fmaf(-lambda, a[MAPS - 1][i] * inv2, o[i]);
         }
     }
-    float f = 1.f;
+    float f = out_scale;
     if (MODE == kFinishDifference) {
         float ss = 0.f;
 #pragma unroll
         for (int i = 0; i < PER_LANE; ++i) ss = fmaf(o[i], o[i], ss);           // (entries beyond dv are zero)
         f = out_scale / sqrtf(wave_sum(ss) / static_cast<float>(dv) + eps);
     }
+    if (MODE == kFinishHeadGate) f *= 1.0f / (1.0f + expf(-gate[static_cast<size_t>(t) * ld_gate + head]));
 #pragma unroll
     for (int i = 0; i < PER_LANE; ++i) {
         const int d = lane + i * kWave;
@@ -313,12 +337,14 @@ using namespace llme;
 
 extern "C" int llme_qk_prepare(const float* p, int ld, int nq, int nk, int nv, int dk, int dv, int k_col, int v_col,
                                const void* wq, const void* wk, int w_dtype, float eps, const float* inv_freq, int rot,
-                               const int* positions, const int* seq_idx, const int* block_table, int max_blocks, void* q_out,
+                               int pairs, float qt_coef, int qt_every, const int* positions, const int* seq_idx, const int* block_table, int max_blocks, void* q_out,
                                int q_dtype, void* k_cache, void* v_cache, int cache_dtype, int page, int T, hipStream_t stream) {
     if (T <= 0) return 0;
-    if (dk <= 0 || dv <= 0 || nv <= 0 || nk % nv != 0 || page <= 0 || rot < 0 || rot > dk || rot % 2 != 0) return kErrBadArgument;
-    if ((wq == nullptr) != (wk == nullptr) || (rot > 0 && inv_freq == nullptr)) return kErrBadArgument;
-    if (v_col < 0 && (nk != nv || dk != dv)) return kErrBadArgument;
+    if (dk <= 0 || page <= 0 || rot < 0 || rot > dk || rot % 2 != 0 || qt_every < 0) return kErrBadArgument;
+    if (nk > 0 && (dv <= 0 || nv <= 0 || nk % nv != 0 || k_cache == nullptr || v_cache == nullptr)) return kErrBadArgument;
+    if (nk == 0) nv = 0;                    // (queries only: the keys and values are another layer's)
+    if ((nk > 0 && (wq == nullptr) != (wk == nullptr)) || (rot > 0 && inv_freq == nullptr)) return kErrBadArgument;
+    if (nk > 0 && v_col < 0 && (nk != nv || dk != dv)) return kErrBadArgument;
     if (dk > kMaxHeadEntries) return kErrBadArgument;
     // enough workgroups for the chip where the step has few tokens: up to a wavefront a head
     const int head_groups = (nq + nk + 3) / 4;
@@ -326,7 +352,7 @@ extern "C" int llme_qk_prepare(const float* p, int ld, int nq, int nk, int nv, i
     const dim3 grid(T, want < head_groups ? (want > 0 ? want : 1) : head_groups);
 #define LLME_PREP(TQ, TC, TW)                                                                                              \
     hipLaunchKernelGGL((qk_prepare_kernel<TQ, TC, TW>), grid, dim3(256), 0, stream, p, ld, nq, nk, nv, dk, dv, k_col, v_col, \
-                       static_cast<const TW*>(wq), static_cast<const TW*>(wk), eps, inv_freq, rot, positions, seq_idx,    \
+                       static_cast<const TW*>(wq), static_cast<const TW*>(wk), eps, inv_freq, rot, pairs, qt_coef, qt_every, positions, seq_idx, \
                        block_table, max_blocks, static_cast<TQ*>(q_out), static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), page)
     if (q_dtype != cache_dtype) return kErrBadArgument;
     if (q_dtype == kF32 && w_dtype == kF32) LLME_PREP(float, float, float);
@@ -340,7 +366,8 @@ extern "C" int llme_qk_prepare(const float* p, int ld, int nq, int nk, int nv, i
 extern "C" int llme_window_attention(const void* q, int q_dtype, const void* k_cache, const void* v_cache, int cache_dtype,
                                      float* part_o, float* part_ml, const int* positions, const int* seq_idx,
                                      const int* block_table, int max_blocks, int T, int nq, int nk, int nv, int dk, int dv, int page,
-                                     float scale, float softcap, int window, int keep_first, hipStream_t stream) {
+                                     float scale, float softcap, int window, int keep_first, const float* slopes,
+                                     hipStream_t stream) {
     if (T <= 0) return 0;
     if (dk <= 0 || dk > kMaxHeadEntries || dv <= 0 || dv > kMaxHeadEntries || nv <= 0 || nk % nv != 0 || page <= 0) return kErrBadArgument;
     const int maps = nk / nv;
@@ -353,12 +380,12 @@ extern "C" int llme_window_attention(const void* q, int q_dtype, const void* k_c
             hipLaunchKernelGGL((window_attention_kernel<TQ, TC, 8>), grid, dim3(8 * 64), 0, stream,                \
                                static_cast<const TQ*>(q), static_cast<const TC*>(k_cache), static_cast<const TC*>(v_cache), \
                                part_o, part_ml, positions, seq_idx, block_table, max_blocks, nq, nk, nv, maps, dk, dv, page, \
-                               scale, softcap, window, keep_first);                                                \
+                               scale, softcap, window, keep_first, slopes);                                              \
         else                                                                                                       \
             hipLaunchKernelGGL((window_attention_kernel<TQ, TC, 1>), grid, dim3(64), 0, stream,                    \
                                static_cast<const TQ*>(q), static_cast<const TC*>(k_cache), static_cast<const TC*>(v_cache), \
                                part_o, part_ml, positions, seq_idx, block_table, max_blocks, nq, nk, nv, maps, dk, dv, page, \
-                               scale, softcap, window, keep_first);                                                \
+                               scale, softcap, window, keep_first, slopes);                                              \
     } while (0)
     if (q_dtype == kF32 && cache_dtype == kF32) LLME_WATT(float, float);
     else if (q_dtype == kBF16 && cache_dtype == kBF16) LLME_WATT(bf16, bf16);
@@ -369,20 +396,22 @@ extern "C" int llme_window_attention(const void* q, int q_dtype, const void* k_c
 
 extern "C" int llme_window_attention_finish(const float* part_o, const float* part_ml, int runs, int T, int heads, int maps, int dv,
                                             int mode, const float* gate, int ld_gate, float lambda, float eps, float out_scale,
-                                            void* out, int out_dtype, int ld_out, hipStream_t stream) {
+                                            const float* sinks, void* out, int out_dtype, int ld_out, hipStream_t stream) {
     if (T <= 0) return 0;
     if (runs <= 0 || heads <= 0 || maps <= 0 || dv <= 0 || dv > kMaxHeadEntries) return kErrBadArgument;
     if ((mode == kFinishDifference && maps != 2) || (mode != kFinishDifference && maps != 1)) return kErrBadArgument;
-    if (mode == kFinishGate && gate == nullptr) return kErrBadArgument;
+    if ((mode == kFinishGate || mode == kFinishHeadGate) && gate == nullptr) return kErrBadArgument;
+    if (sinks != nullptr && maps != 1) return kErrBadArgument;
     const dim3 grid(static_cast<unsigned>((static_cast<size_t>(T) * heads + 3) / 4));
 #define LLME_FIN(TO, MODE)                                                                                            \
     hipLaunchKernelGGL((window_attention_finish_kernel<TO, MODE>), grid, dim3(256), 0, stream, part_o, part_ml, runs, T, heads, \
-                       maps, dv, gate, ld_gate, lambda, eps, out_scale, static_cast<TO*>(out), ld_out)
+                       maps, dv, gate, ld_gate, lambda, eps, out_scale, sinks, static_cast<TO*>(out), ld_out)
 #define LLME_FIN_T(TO)                                                     \
     do {                                                                   \
         if (mode == kFinishPlain) LLME_FIN(TO, kFinishPlain);              \
         else if (mode == kFinishGate) LLME_FIN(TO, kFinishGate);           \
         else if (mode == kFinishDifference) LLME_FIN(TO, kFinishDifference); \
+        else if (mode == kFinishHeadGate) LLME_FIN(TO, kFinishHeadGate);   \
         else return kErrBadArgument;                                       \
     } while (0)
     if (out_dtype == kF32) LLME_FIN_T(float);

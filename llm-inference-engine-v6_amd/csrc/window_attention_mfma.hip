@@ -13,7 +13,8 @@
 // The rows of a 16-key half are laid so that lane l ends up, for query row l % 16, with the scores of the 8 consecutive
 // keys 8 (l / 16) .. of the block: exactly the keys it supplies as second operand of the second product (one 16-byte
 // piece of a value row a tile), so weights never leave their registers. A weight is 32-bit; it enters the second
-// product as the sum of two bfloat16 parts (16 bits of mantissa), and the row's sum adds the 32-bit weights. Blocks
+// product as the sum of two bfloat16 parts (16 bits of mantissa), and the row's sum adds the 32-bit weights. A score may
+// be capped, or lose slope_h x (position - key) (`slopes`, one number a head). Blocks
 // that every row of the tile sees whole (most of a window) skip the tests of visibility. Operands come straight from
 // the pages (no LDS), the next block's keys asked for while this block's weights are made: the four wavefronts of a
 // workgroup take tiles next to each other and find each other's keys in the cache.
@@ -37,7 +38,11 @@ struct WindowArgs {
     const int* block_table;
     int max_blocks, T, nq, nk, nv, maps, per_value_head, dk, dv, page, page_shift, window, keep_first, nsplit;
     float scale, softcap;
+    const float* slopes;        // [nq / maps] or null: a score loses slope (position - key)
 };
+
+// What is done to a raw score besides the scale: nothing, a cap, or a bias that grows with the distance.
+enum ScoreMode : int { kScorePlain = 0, kScoreCapped = 1, kScoreDistance = 2 };
 
 // A capped score from the raw product: cap tanh(scale s / cap) = cap - 2 cap / (e^(2 scale s / cap) + 1), with the
 // hardware's 32-bit power of two and reciprocal; `k` is 2 scale log2(e) / cap. (Where the score is near zero the
@@ -50,15 +55,16 @@ __device__ __forceinline__ float capped_score(float s, float k, float cap) {
 // One block of 32 keys for a tile: scores in sc (this lane's row, keys key0 + 8 qd + j for j = 4 sub + e), values in vf.
 // EDGE: some row of the tile does not see some key of the block (the window's start, the diagonal, kept tokens, rows
 // beyond the request), or a key lies behind the tile's last; otherwise every weight counts and no test is made.
-template <int NVM, bool EDGE, bool CAP>
+template <int NVM, bool EDGE, int CAP>
 __device__ __forceinline__ void window_block(const WindowArgs& a, const f32x4 (&sc)[2], bf16x8 (&vf)[NVM], f32x4 (&acc)[NVM], float& m,
-                                             float& l, int nvt, int key0, int qd, int pos, int pos_max, bool valid, float inv_cap) {
+                                             float& l, int nvt, int key0, int qd, int pos, int pos_max, bool valid, float inv_cap, float slope) {
     float p[8];
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const float v0 = sc[j >> 2][j & 3];
-        float v = CAP ? capped_score(v0, inv_cap, a.softcap) : v0 * a.scale;
+        float v = CAP == kScoreCapped ? capped_score(v0, inv_cap, a.softcap) : v0 * a.scale;
+        if (CAP == kScoreDistance) v = fmaf(slope, static_cast<float>(key0 + qd * 8 + j - pos), v);
         if (EDGE) {
             const int key = key0 + qd * 8 + j;
             const bool seen = valid && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
@@ -108,7 +114,7 @@ __device__ __forceinline__ void window_block(const WindowArgs& a, const f32x4 (&
 }
 
 // DSM, NVM: 32-entry slabs of a key, 16-entry tiles of a value: the most this instance holds. CAP: scores are capped.
-template <int DSM, int NVM, bool CAP>
+template <int DSM, int NVM, int CAP>
 __global__ __launch_bounds__(256, (DSM <= 2 && NVM <= 4) ? 4 : NVM <= 4 ? 3 : 2) void window_attention_mfma_kernel(WindowArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, qd = lane >> 4;
@@ -131,6 +137,7 @@ __global__ __launch_bounds__(256, (DSM <= 2 && NVM <= 4) ? 4 : NVM <= 4 ? 3 : 2)
     const int ds = (a.dk + 31) >> 5, nvt = a.dv >> 4;
     const int psh = a.page_shift, pmask = a.page - 1;
     const float inv_cap = a.softcap > 0.f ? 2.0f * 1.4426950408889634f * a.scale / a.softcap : 0.f;     // (capped_score's k)
+    const float slope = CAP == kScoreDistance ? a.slopes[qh / a.maps] : 0.f;
 
     bf16x8 qf[DSM];
     {
@@ -215,8 +222,8 @@ __global__ __launch_bounds__(256, (DSM <= 2 && NVM <= 4) ? 4 : NVM <= 4 ? 3 : 2)
         // every row sees every key of the block: behind the window's start of the tile's last row, up to the tile's
         // first position, not among the kept blocks (whose keys may lie beyond keep_first)
         const bool inner = all_valid && b >= nb_kept && key0 + 31 <= pos_min && (a.window <= 0 || pos_max - key0 < a.window);
-        if (inner) window_block<NVM, false, CAP>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
-        else window_block<NVM, true, CAP>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap);
+        if (inner) window_block<NVM, false, CAP>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap, slope);
+        else window_block<NVM, true, CAP>(a, sc, vf, acc, m, l, nvt, key0, qd, pos, pos_max, valid, inv_cap, slope);
     }
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -242,15 +249,16 @@ __global__ __launch_bounds__(256, (DSM <= 2 && NVM <= 4) ? 4 : NVM <= 4 ? 3 : 2)
 // only in blocks that some row of its tile does not see whole. Values behind the workgroup's last key are zeroed as
 // they are staged (their page may hold anything). Results are left as by the kernel above, block by block in the same
 // order.
-template <int NVM, bool EDGE, bool CAP>
+template <int NVM, bool EDGE, int CAP>
 __device__ __forceinline__ void shared_block(const WindowArgs& a, const f32x4 (&sc)[2], const bf16* lds_v, f32x4 (&acc)[NVM], float& m,
-                                             float& l, int nvt, int key0, int r, int qd, int pos, bool valid, float inv_cap) {
+                                             float& l, int nvt, int key0, int r, int qd, int pos, bool valid, float inv_cap, float slope) {
     float p[8];
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const float v0 = sc[j >> 2][j & 3];
-        float v = CAP ? capped_score(v0, inv_cap, a.softcap) : v0 * a.scale;
+        float v = CAP == kScoreCapped ? capped_score(v0, inv_cap, a.softcap) : v0 * a.scale;
+        if (CAP == kScoreDistance) v = fmaf(slope, static_cast<float>(key0 + qd * 8 + j - pos), v);
         if (EDGE) {
             const int key = key0 + qd * 8 + j;
             const bool seen = valid && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
@@ -291,7 +299,7 @@ __device__ __forceinline__ void shared_block(const WindowArgs& a, const f32x4 (&
     }
 }
 
-template <int DSM, int NVM, bool CAP>
+template <int DSM, int NVM, int CAP>
 __global__ __launch_bounds__(256, 4) void window_attention_mfma_shared_kernel(WindowArgs a) {
     constexpr int DKP = DSM * 32 + 8;                       // a staged key's stride (entries): 16 bytes of padding
     constexpr int K_ELEMS = 32 * DKP, V_ELEMS = NVM * 16 * 32;
@@ -325,6 +333,7 @@ __global__ __launch_bounds__(256, 4) void window_attention_mfma_shared_kernel(Wi
     const int ds = (a.dk + 31) >> 5, nvt = a.dv >> 4;
     const int psh = a.page_shift, pmask = a.page - 1;
     const float inv_cap = a.softcap > 0.f ? 2.0f * 1.4426950408889634f * a.scale / a.softcap : 0.f;     // (capped_score's k)
+    const float slope = CAP == kScoreDistance ? a.slopes[qh / a.maps] : 0.f;
 
     bf16x8 qf[DSM];
     {
@@ -444,8 +453,8 @@ __global__ __launch_bounds__(256, 4) void window_attention_mfma_shared_kernel(Wi
                 }
             }
             const bool inner = all_valid && b >= nb_kept && key0 + 31 <= pos_min && (a.window <= 0 || pos_max - key0 < a.window);
-            if (inner) shared_block<NVM, false, CAP>(a, sc, lk + K_ELEMS, acc, m, l, nvt, key0, r, qd, pos, valid, inv_cap);
-            else shared_block<NVM, true, CAP>(a, sc, lk + K_ELEMS, acc, m, l, nvt, key0, r, qd, pos, valid, inv_cap);
+            if (inner) shared_block<NVM, false, CAP>(a, sc, lk + K_ELEMS, acc, m, l, nvt, key0, r, qd, pos, valid, inv_cap, slope);
+            else shared_block<NVM, true, CAP>(a, sc, lk + K_ELEMS, acc, m, l, nvt, key0, r, qd, pos, valid, inv_cap, slope);
         }
         if (b + 1 < b_end) stage(buf ^ 1);
         __syncthreads();
@@ -473,11 +482,14 @@ using namespace llme;
 extern "C" int llme_window_attention_mfma(const void* q, const void* k_cache, const void* v_cache, float* part_o, float* part_ml,
                                           const int* positions, const int* q_start, const int* block_table, int max_blocks, int T,
                                           int S, int max_new, int nq, int nk, int nv, int dk, int dv, int page, float scale,
-                                          float softcap, int window, int keep_first, int nsplit, int staged, hipStream_t stream) {
+                                          float softcap, int window, int keep_first, int nsplit, int staged, const float* slopes,
+                                          hipStream_t stream) {
     if (T <= 0 || S <= 0) return 0;
     if (nv <= 0 || nk % nv != 0 || nq % nk != 0 || max_new <= 0 || nsplit <= 0 || window < 0 || keep_first < 0) return kErrBadArgument;
     if (dk % 8 != 0 || dk > 128 || dv % 16 != 0 || dv > 128 || page % 16 != 0 || (page & (page - 1)) != 0) return kErrUnsupported;
+    if (softcap > 0.f && slopes != nullptr) return kErrUnsupported;         // (capped and biased scores: the plain kernel)
     WindowArgs a;
+    a.slopes = slopes;
     a.q = static_cast<const bf16*>(q);
     a.k_cache = static_cast<const bf16*>(k_cache);
     a.v_cache = static_cast<const bf16*>(v_cache);
@@ -506,13 +518,15 @@ extern "C" int llme_window_attention_mfma(const void* q, const void* k_cache, co
     const dim3 grid((tiles + 3) / 4, S * nk, nsplit);
 #define LLME_WMFMA(DSM, NVM)                                                                                     \
     do {                                                                                                         \
-        if (softcap > 0.f) hipLaunchKernelGGL((window_attention_mfma_kernel<DSM, NVM, true>), grid, dim3(256), 0, stream, a); \
-        else hipLaunchKernelGGL((window_attention_mfma_kernel<DSM, NVM, false>), grid, dim3(256), 0, stream, a);  \
+        if (softcap > 0.f) hipLaunchKernelGGL((window_attention_mfma_kernel<DSM, NVM, kScoreCapped>), grid, dim3(256), 0, stream, a); \
+        else if (slopes != nullptr) hipLaunchKernelGGL((window_attention_mfma_kernel<DSM, NVM, kScoreDistance>), grid, dim3(256), 0, stream, a); \
+        else hipLaunchKernelGGL((window_attention_mfma_kernel<DSM, NVM, kScorePlain>), grid, dim3(256), 0, stream, a);  \
     } while (0)
 #define LLME_WSHARED(DSM, NVM)                                                                                          \
     do {                                                                                                                \
-        if (softcap > 0.f) hipLaunchKernelGGL((window_attention_mfma_shared_kernel<DSM, NVM, true>), grid, dim3(256), 0, stream, a); \
-        else hipLaunchKernelGGL((window_attention_mfma_shared_kernel<DSM, NVM, false>), grid, dim3(256), 0, stream, a);  \
+        if (softcap > 0.f) hipLaunchKernelGGL((window_attention_mfma_shared_kernel<DSM, NVM, kScoreCapped>), grid, dim3(256), 0, stream, a); \
+        else if (slopes != nullptr) hipLaunchKernelGGL((window_attention_mfma_shared_kernel<DSM, NVM, kScoreDistance>), grid, dim3(256), 0, stream, a); \
+        else hipLaunchKernelGGL((window_attention_mfma_shared_kernel<DSM, NVM, kScorePlain>), grid, dim3(256), 0, stream, a);  \
     } while (0)
     // a request that brings a workgroup's 64 rows or more, values of up to 64 entries: the blocks staged once a workgroup;
     // fewer rows (decoded tokens, short portions): a wavefront on its own

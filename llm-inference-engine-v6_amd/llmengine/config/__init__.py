@@ -3,11 +3,12 @@ from .llama import LlamaConfig, RopeScaling
 from .rilonex import RilonexConfig
 from .bidirax import BidiraxConfig
 from .zetonex import ZetonexConfig
+from .zapolorn import ZapolornConfig
 from .registry import (Architecture, architecture_name, known_architectures, load_config,
                        parse_config, register_architecture, resolve)
 
 __all__ = [
-    "ConfigError", "KeyReader", "read_model_json", "LlamaConfig", "RopeScaling", "RilonexConfig", "BidiraxConfig", "ZetonexConfig", "Architecture",
+    "ConfigError", "KeyReader", "read_model_json", "LlamaConfig", "RopeScaling", "RilonexConfig", "BidiraxConfig", "ZetonexConfig", "ZapolornConfig", "Architecture",
     "architecture_name", "known_architectures", "load_config", "parse_config",
     "register_architecture", "resolve",
 ]

@@ -71,7 +71,9 @@ class DecoderModel(Part):
         # A tied head is the embedding table under a second name (src/weights.cpp:244-267): a
         # checkpoint may store it under both, and then both must agree in shape and type.
         if getattr(self.head, "tied_to", None) is self.embedding:
-            return {f"{self.names['head']}.weight": f"{self.names['embedding']}.weight"}
+            from ..parts.base import join_name
+            return {join_name(self.names["head"] + ".", getattr(self.head, "tensor", "weight")):
+                    join_name(self.names["embedding"] + ".", getattr(self.embedding, "tensor", "weight"))}
         return {}
 
     # ---- caches ----
@@ -140,6 +142,7 @@ class DecoderModel(Part):
                 layer.next_block = self.layers[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
             layer.forward(h, step, caches[call.cache_id], call.write_cache)
         step.extra.pop("block.normed is for", None)
+        step.extra.pop("block.stream_copy is for", None)
         if logit_rows is None or logit_rows.shape[0] == 0:
             return None
         R = logit_rows.shape[0]

@@ -11,7 +11,7 @@ from .mfma import (gemm_bf16, gemm_gated, gemm_gated_extra, gemm_qkv_rope, gemm_
 
 from . import recurrent                              # noqa: E402
 from .recurrent import (GATE_ACTIVATIONS, copy_cols, delta_gates, delta_rule, gated_activation, gated_head_norm, rglru_gates, rglru_scan,
-                        rotate_write, short_conv, sigmoid_attention, sigmoid_attention_fits, streams_read_norm, streams_spread,
+                        rotate_write, short_conv, sigmoid_attention, sigmoid_attention_fits, sigmoid_decay, streams_read_norm, streams_spread,
                         streams_write, streams_write_read_norm, unit_heads)
 
 from . import latent                                 # noqa: E402
@@ -20,7 +20,7 @@ from .latent import (head_gemm, latent_attention, latent_attention_fits, latent_
 
 from . import window                                 # noqa: E402
 
-__all__ = ["window", "latent", "head_gemm", "latent_attention", "latent_attention_fits", "latent_prepare", "latent_q_rotate", "moe_capacity",
+__all__ = ["window", "sigmoid_decay", "latent", "head_gemm", "latent_attention", "latent_attention_fits", "latent_prepare", "latent_q_rotate", "moe_capacity",
            "moe_combine", "moe_gemm", "moe_plan", "moe_route", "norm_add", "scale_", "GATE_ACTIVATIONS", "copy_cols", "delta_gates", "delta_rule", "gated_activation", "gated_head_norm", "rglru_gates", "rglru_scan",
            "rotate_write", "short_conv", "sigmoid_attention", "sigmoid_attention_fits", "streams_read_norm", "streams_spread",
            "streams_write", "streams_write_read_norm", "unit_heads", "recurrent", "KernelChoices", "ATTENTION_MAX_HEAD_DIM", "gemm_bf16", "gemm_gated", "gemm_gated_extra", "gemm_qkv_rope", "gemm_qkv_rope_supported", "gemv_norm_rope", "gemv_norm_rope_supported", "pair_rows_for_rotation", "gemv_norm", "gemv_norm_supported", "mfma", "KernelError", "KernelLibraryError", "library", "load_kernels", "argmax", "argmax_into", "attention", "attention_generic", "attention_project", "rope_q_only", "embed_gather", "block_weight", "can_block", "clear",

@@ -21,7 +21,7 @@ declare("llme_latent_prepare", [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _f, 
 declare("llme_latent_q_rotate", [_vp, _i, _vp, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp])
 declare("llme_head_gemm", [_vp, _i, _l, _l, _vp, _i, _vp, _i, _l, _l, _i, _i, _i, _i, _vp])
 declare("llme_latent_attention", [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp])
-declare("llme_moe_route", [_vp, _i, _i, _i, _f, _i, _vp, _vp, _vp])
+declare("llme_moe_route", [_vp, _i, _i, _i, _f, _i, _i, _vp, _vp, _vp])
 declare("llme_moe_plan", [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp])
 declare("llme_moe_gemm", [_vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp])
 declare("llme_moe_combine", [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp])
@@ -30,18 +30,19 @@ declare("llme_moe_combine", [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp])
 # --- sandwich norm ---------------------------------------------------------------------
 def norm_add(y: torch.Tensor, w_post: torch.Tensor, h: torch.Tensor, eps: float, w_next: torch.Tensor | None = None,
              x_out: torch.Tensor | None = None) -> None:
-    """h += w_post * y / rms(y); with w_next also x_out = w_next * h / rms(h) of the updated rows.
-    y, h [T, H] 32-bit; the weights multiply as they are."""
+    """h += w_post * y / rms(y); with w_next also x_out = w_next * h / rms(h) of the updated rows; with x_out and no
+    w_next, x_out = the updated rows as they are, in x_out's type. y, h [T, H] 32-bit; the weights multiply as they are."""
     require(y, "y", torch.float32, (None, None))
     T, H = y.shape
     require(h, "h", torch.float32, (T, H))
     require(w_post, "w_post", _FLOATS, (H,))
     if w_next is not None:
         require(w_next, "w_next", w_post.dtype, (H,))
+    if w_next is not None or x_out is not None:
         require(x_out, "x_out", _FLOATS, (T, H))
     check(entry("llme_norm_add")(ptr(y), ptr(w_post), code(w_post.dtype), ptr(h), ptr(w_next),
-                                 code(w_next.dtype) if w_next is not None else 0, ptr(x_out) if w_next is not None else None,
-                                 code(x_out.dtype) if w_next is not None else 0, T, H, float(eps), stream()), "norm_add")
+                                 code(w_next.dtype) if w_next is not None else 0, ptr(x_out),
+                                 code(x_out.dtype) if x_out is not None else 0, T, H, float(eps), stream()), "norm_add")
 
 
 def scale_(x: torch.Tensor, s: float) -> None:
@@ -272,12 +273,18 @@ def moe_capacity(pairs: int, experts: int, tile: int = MOE_TILE) -> int:
     return (pairs + experts * (tile - 1) + tile - 1) // tile * tile
 
 
-def moe_route(logits: torch.Tensor, top: int, scale: float, renormalize: bool, ids: torch.Tensor, wts: torch.Tensor) -> None:
+def moe_route(logits: torch.Tensor, top: int, scale: float, renormalize: bool, ids: torch.Tensor, wts: torch.Tensor,
+              scoring: str = "softmax") -> None:
+    """ids, wts [T, top]: every row's `top` experts with the largest scores, softmax over the row or ("sigmoid") a
+    sigmoid of each logit, and their weights score * scale (over the chosen scores' sum first where `renormalize`)."""
+    if scoring not in ("softmax", "sigmoid"):
+        raise KernelError(f"moe_route: scoring {scoring!r} is neither 'softmax' nor 'sigmoid'")
     require(logits, "logits", torch.float32, (None, None))
     T, E = logits.shape
     require(ids, "ids", torch.int32, (T, top))
     require(wts, "wts", torch.float32, (T, top))
-    check(entry("llme_moe_route")(ptr(logits), T, E, top, float(scale), 1 if renormalize else 0, ptr(ids), ptr(wts), stream()),
+    check(entry("llme_moe_route")(ptr(logits), T, E, top, float(scale), 1 if renormalize else 0, 1 if scoring == "sigmoid" else 0,
+                                  ptr(ids), ptr(wts), stream()),
           "moe_route")
 
 
@@ -344,11 +351,16 @@ def moe_gemm_clamped(a: torch.Tensor, w: torch.Tensor, group: int, out: torch.Te
     return True
 
 
-def moe_combine(y: torch.Tensor, pair_place: torch.Tensor, wts: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
+def moe_combine(y: torch.Tensor, pair_place: torch.Tensor, wts: torch.Tensor | None, out: torch.Tensor, accumulate: bool,
+                top: int | None = None) -> None:
+    """out[t] (+)= sum_k wts[t, k] y[place of pair (t, k)]; wts None: every one of a token's `top` results counts once."""
     require(out, "out", torch.float32, (None, None))
     T, H = out.shape
-    require(wts, "wts", torch.float32, (T, None))
-    top = wts.shape[1]
+    if wts is not None:
+        require(wts, "wts", torch.float32, (T, None))
+        top = wts.shape[1]
+    elif top is None or top <= 0:
+        raise KernelError("moe_combine: without weights the number of results a token has must be given")
     require(y, "y", torch.float32, (None, H))
     require(pair_place, "pair_place", torch.int32, (T * top,))
     check(entry("llme_moe_combine")(ptr(y), ptr(pair_place), ptr(wts), ptr(out), T, top, H, 1 if accumulate else 0, stream()),

@@ -34,7 +34,8 @@ declare("llme_rglru_scan_chunked", [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, 
 declare("llme_copy_cols", [_vp, _i, _vp, _i, _i, _i, _vp])
 declare("llme_unit_heads", [_vp, _i, _i, _i, _i, _i, _f, _f, _f, _vp])
 declare("llme_delta_gates", [_vp, _i, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp])
-declare("llme_delta_rule", [_vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])
+declare("llme_delta_rule", [_vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp])
+declare("llme_sigmoid_decay", [_vp, _i, _vp, _i, _f, _vp, _i, _i, _vp])
 declare("llme_gated_head_norm", [_vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _f, _f, _vp])
 declare("llme_rotate_write", [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp])
 declare("llme_sigmoid_attention", [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp])
@@ -256,19 +257,34 @@ def delta_gates(b_in: torch.Tensor, a_in: torch.Tensor, a2: torch.Tensor | None,
                                     1 if per_channel else 0, stream()), "delta_gates")
 
 
-def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, step, o: torch.Tensor,
-               heads: int, kv_heads: int, dim: int, vdim: int, per_channel: bool) -> None:
+def sigmoid_decay(z: torch.Tensor, bias: torch.Tensor | None, tau: float, decay: torch.Tensor) -> None:
+    """decay [T, n] (32-bit) = sigmoid(z + bias)^(1 / tau), z [T, n] a column range of a 32-bit buffer."""
+    T, n = z.shape
+    ld = _cols(z, "z", torch.float32, T, n)
+    if bias is not None:
+        require(bias, "bias", _FLOATS, (n,))
+    require(decay, "decay", torch.float32, (T, n))
+    if not tau > 0:
+        raise KernelError(f"sigmoid_decay: tau={tau} must be > 0")
+    check(entry("llme_sigmoid_decay")(ptr(z), ld, ptr(bias), code(bias.dtype) if bias is not None else 0, float(tau), ptr(decay),
+                                      T, n, stream()), "sigmoid_decay")
+
+
+def delta_rule(qkv: torch.Tensor, beta: torch.Tensor | None, decay: torch.Tensor, state: torch.Tensor, step, o: torch.Tensor,
+               heads: int, kv_heads: int, dim: int, vdim: int, per_channel: bool, q_scale: float = 1.0) -> None:
     """The delta rule over each request's rows, from and into its slot of state [slots, heads, vdim, dim] (M transposed:
     a column's key channels lie together):
-    M <- decay * M; w = beta (v - M^T k); M <- M + k w^T; o = M^T q. qkv [T, (2 kv_heads dim + heads vdim)] holds
-    unit q, unit k and v side by side; decay is [T, heads * dim] (per key channel) or [T, heads]."""
+    M <- decay * M; w = beta (v - M^T k); M <- M + k w^T; o = q_scale M^T q. beta None: the linear rule, w = v (nothing
+    is read back before the write). qkv [T, (2 kv_heads dim + heads vdim)] holds q, k and v side by side; decay is
+    [T, heads * dim] (per key channel) or [T, heads]."""
     T = qkv.shape[0]
     ld = _cols(qkv, "qkv", torch.float32, T, 2 * kv_heads * dim + heads * vdim)
     if heads % kv_heads:
         raise KernelError(f"delta_rule: {heads} heads do not divide into {kv_heads} key heads")
     if dim > DELTA_MAX_DIM:
         raise KernelError(f"delta_rule: key size {dim} is beyond the kernel's limit of {DELTA_MAX_DIM}")
-    require(beta, "beta", torch.float32, (T, heads))
+    if beta is not None:
+        require(beta, "beta", torch.float32, (T, heads))
     require(decay, "decay", torch.float32, (T, None))
     if decay.shape[1] != (heads * dim if per_channel else heads):
         raise KernelError(f"delta_rule: decay has {decay.shape[1]} columns for {heads} heads of {dim}")
@@ -278,7 +294,7 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state
         raise KernelError("delta_rule: one row per token of the step")
     check(entry("llme_delta_rule")(ptr(qkv), ld, 0, kv_heads * dim, 2 * kv_heads * dim, ptr(beta), ptr(decay),
                                    1 if per_channel else 0, ptr(state), ptr(step.q_start), ptr(step.slots), ptr(o),
-                                   step.num_seqs, heads, kv_heads, dim, vdim, stream()), "delta_rule")
+                                   step.num_seqs, heads, kv_heads, dim, vdim, float(q_scale), stream()), "delta_rule")
 
 
 def gated_head_norm(o: torch.Tensor, weight: torch.Tensor, gate_in: torch.Tensor, g2: torch.Tensor | None, out: torch.Tensor,

@@ -6,7 +6,7 @@ from .rope import RotaryEmbedding, inverse_frequencies
 from .embedding import Embedding, OutputHead
 from .mlp import GatedMLP
 from .attention import Attention
-from .block import ParallelBlock, PreNormBlock, SandwichBlock
+from .block import OutputNormBlock, ParallelBlock, PreNormBlock, SandwichBlock
 from .projected import ParallelMixer, ProjectedMixer
 from .rglru import RGLRU
 from .delta import GatedDeltaRule
@@ -15,6 +15,7 @@ from .hyper import HyperConnectionBlock
 from .latent_attention import LatentAttention
 from .moe import MixtureOfExperts
 from .window_attention import WindowAttention
+from .linear_attention import GatedLinearAttention
 from .reentry import PassInput
 
 __all__ = ["PAGE", "Block", "CacheSpec", "FeedForward", "LayerCache", "Mixer", "Norm", "ParamSpec", "Part",
@@ -22,4 +23,4 @@ __all__ = ["PAGE", "Block", "CacheSpec", "FeedForward", "LayerCache", "Mixer", "
            "register_part", "registered", "RMSNorm", "RotaryEmbedding", "inverse_frequencies", "Embedding",
            "OutputHead", "GatedMLP", "Attention", "PreNormBlock", "ParallelMixer", "ProjectedMixer", "RGLRU", "GatedDeltaRule",
            "SigmoidAttention", "HyperConnectionBlock", "CenteredRMSNorm", "SandwichBlock", "LatentAttention",
-           "MixtureOfExperts", "WindowAttention", "PassInput", "ParallelBlock"]
+           "MixtureOfExperts", "WindowAttention", "PassInput", "ParallelBlock", "OutputNormBlock", "GatedLinearAttention"]

@@ -139,6 +139,60 @@ class ParallelBlock(Block):
             self.feed_forward.forward(x, step, h, True)
 
 
+class OutputNormBlock(Block):
+    """Norms behind the sublayers only: h += norm1(mixer(h)); h += norm2(ffn(h)). The sublayers read the stream itself
+    (rounded to the activation type where that is not 32-bit); a sublayer's result is a 32-bit buffer of its own, and
+    the norm behind it, the sum into the stream and the copy of the updated rows that the next sublayer reads (this
+    block's feed-forward, or the mixer of the block behind) are one kernel."""
+    graph_safe = True
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward | None, mixer_norm: Norm, ffn_norm: Norm | None,
+                 names: dict | None = None):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.ffn_norm = mixer_norm, ffn_norm
+        self.names = {"mixer_norm": "norm1", "mixer": "mix", "ffn_norm": "norm2", "feed_forward": "mlp"}
+        if names:
+            self.names.update(names)
+        # the block that runs behind this one (told by the model as it runs its schedule; None: unknown)
+        self.next_block = None
+
+    def children(self):
+        n = self.names
+        out = {n["mixer_norm"]: self.mixer_norm, n["mixer"]: self.mixer}
+        if self.feed_forward is not None:
+            out.update({n["ffn_norm"]: self.ffn_norm, n["feed_forward"]: self.feed_forward})
+        return out
+
+    @staticmethod
+    def _join(y, post: Norm, h, x) -> None:
+        """h += post(y), and x = the updated rows where x is another buffer than the stream."""
+        rms = post.fused_rms()
+        if rms is None:
+            raise NotImplementedError("output-norm blocks take norms of the plain RMS formula behind their sublayers")
+        ops.norm_add(y, rms[0], h, rms[1], None, x if x is not h else None)
+
+    def forward(self, h, step, cache, write_cache=True):
+        T, H = h.shape
+        y = step.buffer("block.sublayer", (T, H), torch.float32)
+        if step.act_dtype == torch.float32:
+            x = h                           # (the sublayers read the 32-bit stream as it lies)
+        else:
+            x = step.buffer("block.stream_copy", (T, H), step.act_dtype)
+            if step.extra.pop("block.stream_copy is for", None) != id(self):
+                ops.copy_cols(h, x)
+        self.mixer.forward(x, step, cache, y, False, write_cache)
+        hand_on = isinstance(self.next_block, OutputNormBlock) and x is not h
+        if self.feed_forward is None:
+            self._join(y, self.mixer_norm, h, x if hand_on else h)
+        else:
+            self._join(y, self.mixer_norm, h, x)
+            self.feed_forward.forward(x, step, y, False)
+            self._join(y, self.ffn_norm, h, x if hand_on else h)
+        if hand_on:
+            step.extra["block.stream_copy is for"] = id(self.next_block)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "output_norm", OutputNormBlock)
 register_part("block", "parallel", ParallelBlock)
 register_part("block", "sandwich", SandwichBlock)

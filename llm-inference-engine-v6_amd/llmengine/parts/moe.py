@@ -7,6 +7,10 @@ largest s are chosen (the lower index wins a tie), weight = s * scale, divided b
 first where `renormalize` is set. Expert e: down_e(act(gate_e x) * up_e x), no biases. Tensors: "router",
 "e<i>.gate", "e<i>.up", "e<i>.down"; the shared expert is a child part under "shared".
 
+`router="sigmoid"`: the scores are sigmoid(z), each expert's on its own, and the largest are chosen.
+`weight_on="input"`: a chosen expert runs on weight * x and its result is added as it is (the weight is taken out of
+the expert's two input products: their 32-bit sums are multiplied by it in front of the activation).
+
 `router="table"`: there is no router matrix; a table [vocab, top] of integers ("table"; the entries of a row differ)
 names the experts of every token id, each weighing 1 / top. `activation="swish_clamped"` with `limit`:
 g = min(gate, limit), u = clamp(up, -limit, limit), the expert's inner value is g sigmoid(1.702 g) (u + 1).
@@ -29,9 +33,14 @@ class MixtureOfExperts(FeedForward):
 
     def __init__(self, hidden_size: int, intermediate_size: int, experts: int, top: int, scale: float = 1.0,
                  renormalize: bool = False, activation: str = "silu", shared: FeedForward | None = None,
-                 expert_name: str = "e{}", router: str = "softmax", vocab_size: int = 0, limit: float = 0.0):
-        if router not in ("softmax", "table"):
-            raise ValueError(f"mixture_of_experts: router {router!r} is neither 'softmax' nor 'table'")
+                 expert_name: str = "e{}", router: str = "softmax", vocab_size: int = 0, limit: float = 0.0,
+                 weight_on: str = "output"):
+        if router not in ("softmax", "sigmoid", "table"):
+            raise ValueError(f"mixture_of_experts: router {router!r} is none of 'softmax', 'sigmoid' and 'table'")
+        if weight_on not in ("output", "input"):
+            raise ValueError(f"mixture_of_experts: weight_on {weight_on!r} is neither 'output' nor 'input'")
+        if weight_on == "input" and activation == "swish_clamped":
+            raise ValueError("mixture_of_experts: weights on the experts' input do not go with the clamped activation")
         if router == "table" and vocab_size <= 0:
             raise ValueError("mixture_of_experts: a table of experts by token id needs vocab_size")
         if not 1 <= top <= experts:
@@ -42,6 +51,7 @@ class MixtureOfExperts(FeedForward):
         if activation == "swish_clamped" and not limit > 0:
             raise ValueError("mixture_of_experts: the clamped activation needs limit > 0")
         self.router, self.vocab_size, self.limit = router, int(vocab_size), float(limit)
+        self.weight_on = weight_on
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.experts, self.top, self.scale = int(experts), int(top), float(scale)
         self.renormalize, self.activation = bool(renormalize), activation
@@ -57,7 +67,7 @@ class MixtureOfExperts(FeedForward):
 
     def param_specs(self):
         H, FF = self.hidden_size, self.intermediate_size
-        out = ({"router": ParamSpec((self.experts, H))} if self.router == "softmax"
+        out = ({"router": ParamSpec((self.experts, H))} if self.router != "table"
                else {"table": ParamSpec((self.vocab_size, self.top), f"table:{self.experts}")})
         for e in range(self.experts):
             name = self.expert_name.format(e)
@@ -67,7 +77,7 @@ class MixtureOfExperts(FeedForward):
     def load_params(self, get: Getter, placement: Placement) -> None:
         # The router's matrix as the file has it: bfloat16 entries times the bfloat16 input are exact in 32-bit, so the
         # matrix-core product with its 32-bit sums is the 32-bit product; the 32-bit model widens it like everything else.
-        if self.router == "softmax":
+        if self.router != "table":
             self.w_router = placement.place(get("router"))
         else:
             self.table = placement.place(get("table"))
@@ -95,7 +105,7 @@ class MixtureOfExperts(FeedForward):
         else:
             logits = step.buffer("moe.logits", (T, E), f32)
             ops.gemm(x, self.w_router, logits, choices=step.choices)
-            ops.moe_route(logits, top, self.scale, self.renormalize, ids, wts)
+            ops.moe_route(logits, top, self.scale, self.renormalize, ids, wts, scoring=self.router)
         tile = ops.latent.moe_tile(x, self.w_gate_up, T * top, E, self.group, step.choices)
         cap = ops.moe_capacity(T * top, E, tile)
         place_pair, pair_place = step.buffer("moe.place_pair", (cap,), i32), step.buffer("moe.pair_place", (T * top,), i32)
@@ -106,6 +116,11 @@ class MixtureOfExperts(FeedForward):
                                                                              tile_expert, n_tiles, tile, top, self.limit, 1.702,
                                                                              step.choices):
             pass                            # (clamps and activation in the product's epilogue)
+        elif self.weight_on == "input":
+            # the gate and up sums as 32-bit rows, each row times its pair's weight, then the activation, in one pass
+            gu = step.buffer("moe.gate_up", (cap, 2 * FF), f32)
+            ops.moe_gemm(x, self.w_gate_up, False, 0, gu, place_pair, tile_expert, n_tiles, tile, top, "silu", step.choices)
+            ops.window.gated_bias_act(gu, act, self.group, self.activation, row_pair=place_pair, pair_scale=wts.view(-1))
         elif self.activation == "swish_clamped":
             # the gate and up columns as 32-bit rows, then clamps and activation in one pass
             gu = step.buffer("moe.gate_up", (cap, 2 * FF), f32)
@@ -119,7 +134,7 @@ class MixtureOfExperts(FeedForward):
         if self.shared is not None:
             self.shared.forward(x, step, out, accumulate)
             accumulate = True
-        ops.moe_combine(y, pair_place, wts, out, accumulate)
+        ops.moe_combine(y, pair_place, wts if self.weight_on == "output" else None, out, accumulate, top=top)
 
 
 register_part("feed_forward", "mixture_of_experts", MixtureOfExperts)

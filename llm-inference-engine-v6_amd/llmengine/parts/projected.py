@@ -48,6 +48,7 @@ class ProjectedMixer(Mixer):
     hidden_size: int
     out_width: int                      # columns of the core's result = inputs of the output matrix
     stacked_by_parent = False           # True: a parent stacks this mixer's matrices with others' and runs the products
+    reads_foreign_cache = False         # True: the mixer keeps nothing itself and works on the cache another layer writes
 
     def input_names(self) -> list[tuple[str, int]]:
         """(local tensor name, rows) of the matrices that read the layer's input, in the order of the columns
@@ -78,8 +79,9 @@ class ProjectedMixer(Mixer):
         self.w_out = placement.place_matrix(get(self.output_name()))
 
     def forward(self, x, step, cache, out, accumulate, write_cache=True):
-        if not write_cache:
-            raise NotImplementedError(f"{type(self).__name__} keeps a state of its own and cannot read another layer's")
+        if write_cache == self.reads_foreign_cache:
+            raise NotImplementedError(f"{type(self).__name__} keeps a state of its own and cannot read another layer's"
+                                      if not write_cache else f"{type(self).__name__} has nothing to write into a cache")
         T = x.shape[0]
         p = step.buffer("mixer.projected", (T, self.in_padded), torch.float32)
         ops.gemm(x, self.w_in, p, choices=step.choices)
