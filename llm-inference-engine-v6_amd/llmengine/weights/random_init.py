@@ -66,6 +66,10 @@ def write_random_model(config_dict: dict, out_dir: str, seed: int, dtype: torch.
     arch = resolve(architecture_name(config_dict))
     model = arch.build_model(parse_config(config_dict))
     specs = model.named_specs()
+    for name, spec in specs.items():
+        if any(d is None for d in spec.shape):
+            raise ValueError(f"random weights: the shape of {name} ({tuple(spec.shape)}) has a size that only a checkpoint gives; "
+                             "name it in the configuration")
     os.makedirs(out_dir, exist_ok=True)
     with open(os.path.join(out_dir, "config.json"), "w", encoding="utf-8") as f:
         json.dump(config_dict, f, indent=2)

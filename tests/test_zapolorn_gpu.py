@@ -1,0 +1,421 @@
+"""Zapolorn on the GPU against the plain implementation (tests/plain_zapolorn.py): every mechanism alone and
+together, under every way of cutting requests into steps, in 32-bit and in bfloat16."""
+from __future__ import annotations
+
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+import plain_zapolorn as plain
+import replay
+import zapolorn_models as zm
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 2e-4          # of a row's root mean square; honest 32-bit arithmetic is at 1e-5
+# bfloat16 against the unrounded plain model: narrow models with weights of order one, and experts chosen by scores
+# that rounding swaps now and then (random routers have close calls; the token's row and what later tokens read of it
+# then differ by their whole size: with every expert chosen the same models are at 6e-3 on average and 2e-2 at worst).
+# So half the rows are held tightly and the average loosely; a fault of a kernel moves all rows by their whole size.
+# What a schedule changes is held tightly, against the whole prompts' rows.
+BF16_MEDIAN, BF16_MEAN, BF16_BETWEEN_SCHEDULES = 3e-2, 0.12, 4e-2
+
+
+def _median(got, ref) -> float:
+    return float(np.median(_errors(got, ref)))
+
+
+def _engine(tmp_path, cfg, seed, dtype, weights=None, **kw):
+    from llmengine import Engine
+    store = torch.float32 if dtype == "fp32" else torch.bfloat16
+    folder, weights = zm.write_model(tmp_path, cfg, seed, store, weights)
+    return Engine(folder, dtype, deterministic=True, **kw), weights
+
+
+def _tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def _reference(cfg, weights, requests):
+    w = {k: v.float() for k, v in weights.items()}
+    return {rid: plain.forward(cfg, w, ids).numpy() for rid, ids in requests.items()}
+
+
+def _errors(got: dict, ref: dict) -> list[float]:
+    return [float(np.sqrt(np.mean((row - ref[rid][pos]) ** 2)) / np.sqrt(np.mean(ref[rid][pos] ** 2)))
+            for rid, rows in got.items() for pos, row in rows.items()]
+
+
+def _worst(got, ref) -> float:
+    return max(_errors(got, ref))
+
+
+def _most(got, ref) -> float:
+    return float(np.quantile(_errors(got, ref), 0.97))
+
+
+def _mean(got, ref) -> float:
+    return float(np.mean(_errors(got, ref)))
+
+
+def _covered(got: dict, requests: dict) -> bool:
+    return all(sorted(got[rid]) == list(range(len(ids))) for rid, ids in requests.items())
+
+
+def _stacked(got: dict) -> dict:
+    return {rid: np.stack([rows[p] for p in sorted(rows)]) for rid, rows in got.items()}
+
+
+ONE_LAYER = {
+    "windowed": zm.config([zm.windowed(mlp=None)]),
+    "windowed_sharp": zm.config([zm.windowed(window=9, sharp=6.0, mlp=None)]),
+    "windowed_no_window": zm.config([zm.windowed(window=0, sharp=4.0, mlp=None)]),
+    "windowed_window_of_one": zm.config([zm.windowed(window=1, mlp=None)]),
+    "windowed_no_rotation_one_head": zm.config([zm.windowed(heads=1, kv_heads=1, dim=20, vdim=20, dims=0, window=17, sharp=5.0, mlp=None)]),
+    "windowed_whole_head_rotated_no_factor": zm.config([zm.windowed(heads=6, kv_heads=3, dim=8, vdim=6, dims=8, factor=0, window=8, mlp=None)]),
+    "windowed_wide_heads": zm.config([zm.windowed(heads=2, kv_heads=1, dim=136, vdim=70, dims=70, window=19, scale=0.08, mlp=None)], width=36),
+    "a_reader_with_the_wider_window": zm.config([zm.windowed(window=5, sharp=4.0, mlp=None), zm.windowed(window=12, kv_from=0, sharp=4.0, mlp=None)]),
+    "a_reader_with_the_narrower_window": zm.config([zm.windowed(window=12, sharp=4.0, mlp=None), zm.windowed(window=3, kv_from=0, sharp=4.0, mlp=None)]),
+    "a_reader_without_a_window_and_other_heads": zm.config([zm.windowed(window=6, mlp=None), zm.windowed(heads=2, window=0, kv_from=0, mlp=None)]),
+    "parallel": zm.config([zm.parallel(mlp=None)]),
+    "parallel_sharp_left": zm.config([zm.parallel(sharp=6.0, right_scale=0.2, mlp=None)]),
+    "parallel_right_alone_counts": zm.config([zm.parallel(left_scale=0.05, right_scale=2.0, mlp=None)]),
+    "parallel_no_temperature_one_head": zm.config([zm.parallel(heads=1, kv_heads=1, dim=16, vdim=16, every=0, mlp=None)]),
+    "parallel_temperature_every_token": zm.config([zm.parallel(coef=1.5, every=1, mlp=None)]),
+    "parallel_eight_heads_of_their_own": zm.config([zm.parallel(heads=8, kv_heads=8, dim=4, vdim=4, r_heads=1, r_dim=20, r_vdim=3, mlp=None)]),
+    "parallel_wide_memory": zm.config([zm.parallel(r_heads=1, r_dim=70, r_vdim=40, tau=20.0, rank=3, mlp=None)]),
+    "parallel_fast_forgetting": zm.config([zm.parallel(r_heads=5, r_dim=2, r_vdim=2, tau=0.5, rank=1, mlp=None)]),
+    "dense": zm.config([zm.windowed(mlp="dense")]),
+    "experts_two_of_five_and_a_shared_one": zm.config([zm.parallel(mlp="moe")]),
+    "experts_one_of_three_none_shared": zm.config([zm.windowed(mlp=zm.feed_forward("moe", experts=3, top=1, shared=0))]),
+    "every_expert_chosen": zm.config([zm.windowed(mlp=zm.feed_forward("moe", ff=10, experts=4, top=4))]),
+    "seventy_experts": zm.config([zm.parallel(mlp=zm.feed_forward("moe", ff=6, experts=70, top=5))]),
+    "width_of_30_nothing_scaled": zm.config([zm.windowed(heads=5, kv_heads=5, dim=6, vdim=6, dims=2, mlp=zm.feed_forward("moe", ff=9))], width=30, vocab=33,
+                                            logit_scale=1.0, embedding_scale=1.0),
+}
+
+
+@pytest.mark.parametrize("name", sorted(ONE_LAYER))
+def test_each_mechanism_alone_whole_token_by_token_and_in_portions(tmp_path, name):
+    cfg = ONE_LAYER[name]
+    engine, weights = _engine(tmp_path, cfg, 3, "fp32")
+    requests = {"a": _tokens(41, cfg["vocab"], 1), "b": _tokens(1, cfg["vocab"], 2)}
+    ref = _reference(cfg, weights, requests)
+    for steps in (replay.whole(requests), replay.tail_one_by_one(requests, tail=40), replay.portions(requests),
+                  replay.portions(requests, sizes=(2,))):
+        cache = engine.new_cache(replay.trace_peak_tokens(steps, 8) // 8 + 1, 8, 2)
+        got = replay.run_trace(engine, cache, steps)
+        assert _covered(got, requests)
+        assert _worst(got, ref) < F32_TOL
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("cfg_name", ["MIXED", "ALIGNED"])
+def test_every_schedule_gives_the_plain_logits(tmp_path, cfg_name, dtype):
+    cfg = getattr(zm, cfg_name)
+    engine, weights = _engine(tmp_path, cfg, 11, dtype)
+    V = cfg["vocab"]
+    requests = {"long": _tokens(150, V, 5), "one": _tokens(1, V, 6), "two": _tokens(2, V, 7), "mid": _tokens(49, V, 8),
+                "page": _tokens(32, V, 9), "more": _tokens(65, V, 10)}
+    ref = _reference(cfg, weights, requests)
+    schedules = {
+        "whole": replay.whole(requests),
+        "tail": replay.tail_one_by_one(requests, tail=40),
+        "portions": replay.portions(requests),
+        "portions of two": replay.portions(requests, sizes=(2,)),
+        "mixed": replay.mixed(requests, max_live=3, seed=1),
+        "mixed, other cuts": replay.mixed(requests, max_live=2, sizes=(2, 17, 3, 31), seed=2),
+    }
+    first = None
+    for what, steps in schedules.items():
+        for page in (16, 8):
+            # as many pages as the live requests need and three slots: pages and slots are used again
+            cache = engine.new_cache(replay.trace_peak_tokens(steps, page) // page, page, 3)
+            got = replay.run_trace(engine, cache, steps)
+            assert _covered(got, requests), what
+            if dtype == "fp32":
+                assert _worst(got, ref) < F32_TOL, (what, page)
+            else:
+                assert _median(got, ref) < BF16_MEDIAN and _mean(got, ref) < BF16_MEAN, (what, page)
+                first = first or _stacked(got)
+                assert _most(got, first) < BF16_BETWEEN_SCHEDULES and _mean(got, first) < BF16_BETWEEN_SCHEDULES / 2, (what, page)
+            assert not cache.manager.live_requests()
+
+
+MATRIX_CORES = {
+    # three heads on one key/value head (a wavefront's 16 rows are 5 tokens and a third), key entries of 48 (a slab and a
+    # half), values of 80, a window that ends inside blocks of keys; the left side with five heads on one
+    "three_heads": zm.config([zm.windowed(heads=3, kv_heads=1, dim=48, vdim=80, dims=24, window=37, scale=0.12, sharp=3.0, mlp=None),
+                              zm.parallel(heads=5, kv_heads=1, dim=48, vdim=16, scale=0.15, every=7, sharp=3.0, mlp=None),
+                              zm.windowed(heads=6, kv_heads=1, dim=48, vdim=80, dims=24, window=70, kv_from=0, scale=0.12, sharp=3.0, mlp=None)],
+                             width=32),
+    # every head with keys of its own (a tile holds one head of 16 tokens), heads of 16 and of 128
+    "heads_of_their_own": zm.config([zm.windowed(heads=4, kv_heads=4, dim=16, vdim=32, dims=16, window=50, scale=0.2, sharp=3.0, mlp=None),
+                                     zm.parallel(heads=2, kv_heads=2, dim=128, vdim=128, scale=0.09, every=100, sharp=3.0, mlp=None)], width=32),
+    # 24 heads on two key/value heads (a token's heads fill a tile and a half), no window, and a window of 130
+    "many_heads": zm.config([zm.windowed(heads=24, kv_heads=2, dim=32, vdim=16, dims=8, window=0, scale=0.15, sharp=3.0, mlp=None),
+                             zm.parallel(heads=16, kv_heads=2, dim=32, vdim=32, scale=0.15, every=33, sharp=2.0, mlp=None),
+                             zm.windowed(heads=8, kv_heads=1, dim=64, vdim=64, dims=32, window=130, scale=0.1, sharp=3.0, mlp=None)],
+                            width=32),
+}
+
+
+@pytest.mark.parametrize("name", sorted(MATRIX_CORES))
+def test_the_matrix_core_attention_at_other_sizes(tmp_path, name):
+    """bfloat16 on the matrix cores against the same model on the plain-precision kernels (what differs is the order of
+    sums), under every schedule, and both against the plain model."""
+    from llmengine.ops import KernelChoices
+    cfg = MATRIX_CORES[name]
+    engine, weights = _engine(tmp_path, cfg, 21, "bf16")
+    slow_engine, _ = _engine(tmp_path / "plain", cfg, 21, "bf16", weights=weights, kernel_choices=KernelChoices(fast_attention=False))
+    V = cfg["vocab"]
+    requests = {"a": _tokens(300, V, 1), "b": _tokens(21, V, 2), "c": _tokens(1, V, 3)}
+    ref = _reference(cfg, weights, requests)
+    slow = _stacked(replay.run_trace(slow_engine, slow_engine.new_cache(32, 16, 3), replay.whole(requests)))
+    for steps in (replay.whole(requests), replay.tail_one_by_one(requests, tail=150), replay.portions(requests, sizes=(33, 2, 64, 7, 1, 41)),
+                  replay.mixed(requests, max_live=3, sizes=(50, 3, 24, 2), seed=4)):
+        got = replay.run_trace(engine, engine.new_cache(replay.trace_peak_tokens(steps, 16) // 16, 16, 3), steps)
+        assert _covered(got, requests)
+        assert _mean(got, slow) < 1e-2 and _most(got, slow) < 3e-2
+        assert _mean(got, ref) < 6e-2
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_a_batch_of_unequal_requests_against_each_alone(tmp_path, dtype):
+    cfg = zm.ALIGNED
+    engine, _ = _engine(tmp_path, cfg, 12, dtype)
+    V = cfg["vocab"]
+    requests = {"a": _tokens(70, V, 1), "b": _tokens(3, V, 2), "c": _tokens(1, V, 3), "d": _tokens(33, V, 4)}
+    alone = _stacked(replay.run_trace(engine, engine.new_cache(8, 16, 1), replay.whole(requests)))
+    together = [{"step": 0, "entries": [{"id": r, "tokens": ids, "want": list(range(len(ids)))} for r, ids in requests.items()],
+                 "end": list(requests)}]
+    got = replay.run_trace(engine, engine.new_cache(12, 16, 4), together)
+    assert _worst(got, alone) < (1e-5 if dtype == "fp32" else 2e-2)
+
+
+def test_a_slot_that_is_used_again_starts_from_an_empty_memory(tmp_path):
+    """One state slot: the second request takes the slot the first one left, and must not find its memory there."""
+    cfg = zm.config([zm.parallel(left_scale=0.05, right_scale=2.0, tau=30.0, mlp=None)])
+    engine, weights = _engine(tmp_path, cfg, 5, "fp32")
+    requests = {"first": _tokens(40, cfg["vocab"], 1), "second": _tokens(25, cfg["vocab"], 2)}
+    ref = _reference(cfg, weights, requests)
+    cache = engine.new_cache(4, 16, 1)
+    for steps in (replay.whole(requests), replay.portions(requests, sizes=(9, 2)), replay.tail_one_by_one(requests, tail=10)):
+        got = replay.run_trace(engine, cache, steps)
+        assert _worst(got, ref) < F32_TOL
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_far_keys_page_borders_and_window_edges(tmp_path, dtype):
+    """Sharp softmaxes over a long prompt: the layers without a window find their keys anywhere among hundreds (the bias by
+    distance decides between far and near ones), the windowed layers stand on keys just inside their windows (40 and 24
+    tokens: edges inside pages, at page borders and across them as the prompt moves along), the temperature of the
+    queries steps many times, and the memory carries over hundreds of tokens; in prompts cut anywhere and in decoding
+    far behind the window's first pass."""
+    cfg = copy.deepcopy(zm.ALIGNED)
+    for layer, sharp in zip(cfg["layers"], (3.0, 3.5, 3.5, 3.0)):
+        m = layer["mixer"]
+        (m["left"] if "left" in m else m)["scale"] *= sharp
+    engine, weights = _engine(tmp_path, cfg, 13, dtype)
+    V = cfg["vocab"]
+    requests = {"far": _tokens(700, V, 1), "edge": _tokens(90, V, 2)}
+    ref = _reference(cfg, weights, requests)
+    schedules = [replay.whole(requests), replay.tail_one_by_one(requests, tail=70), replay.portions(requests, sizes=(33, 2, 64, 7, 16, 1, 41)),
+                 replay.mixed(requests, max_live=2, prompt_frac=0.8, sizes=(50, 3, 24, 2), seed=4)]
+    first = None
+    for steps in schedules:
+        cache = engine.new_cache(replay.trace_peak_tokens(steps, 16) // 16, 16, 2)
+        got = replay.run_trace(engine, cache, steps)
+        assert _covered(got, requests)
+        if dtype == "fp32":
+            assert _worst(got, ref) < 2 * F32_TOL       # (scores several times larger carry their rounding into the weights)
+        else:
+            assert _mean(got, ref) < 6e-2
+            first = first or _stacked(got)
+            assert np.mean(_errors(got, first)) < 2e-2
+
+
+def _hand_made(kind: str):
+    """A single layer whose scores are made by hand: a query of token id 1 scores a key of id 2 far above all others and
+    the key's value moves the row. Queries and keys are normed per head, so what singles the key out is its direction:
+    the key matrix spreads ordinary tokens over many entries and id 2 over one."""
+    D = 16
+    if kind == "windowed":
+        cfg = zm.config([zm.windowed(heads=1, kv_heads=1, dim=D, vdim=D, dims=0, window=24, scale=2.0, mlp=None)], width=D, vocab=9,
+                        embedding_scale=1.0)
+        pre = "l0.mix."
+    else:
+        cfg = zm.config([zm.parallel(heads=1, kv_heads=1, dim=D, vdim=D, scale=2.0, every=0, left_scale=1.0, right_scale=0.0, mlp=None)],
+                        width=D, vocab=9, embedding_scale=1.0)
+        pre = "l0.mix.left."
+    weights = zm.make_weights(cfg, 31, torch.float32)
+    wk = torch.eye(D)
+    wk[0, 0], wk[0, 1], wk[1, 1], wk[3, 3] = 0.0, 1.0, 0.0, 0.0      # a key's entry 0 is the stream's entry 1
+    wv = torch.zeros(D, D)
+    wv[3, 3] = 1.0                                                   # a value carries the stream's entry 3
+    weights[pre + "q"], weights[pre + "k"], weights[pre + "v"] = torch.eye(D), wk, wv
+    weights[pre + "q.norm"], weights[pre + "k.norm"] = torch.ones(D), torch.ones(D)
+    if kind == "windowed":
+        weights["l0.mix.sink"] = torch.zeros(1)
+        weights["l0.mix.g"] = torch.zeros(1, D)
+    weights["embed"] = torch.randn(9, D, generator=torch.Generator().manual_seed(5)) * 0.3
+    weights["embed"][:, 3] = 0
+    weights["embed"][1] = 0
+    weights["embed"][1, 0] = 6.0
+    weights["embed"][2] = 0
+    weights["embed"][2, 1] = 5.0
+    weights["embed"][2, 3] = 4.0                    # what the row carries when the key is seen
+    return cfg, weights
+
+
+def test_one_key_stands_out_far_back_and_at_the_window_edge(tmp_path):
+    """Where the one key lies (on the window's edge, one token outside it, at a page border; far back where there is no
+    window) decides the row; the engine follows the plain model in each place, in a prompt and decoded."""
+    fill = [3, 4, 5, 6, 7, 8]
+    base = [fill[i % 6] for i in range(200)]
+    for kind, places in (("windowed", (("window edge", 199 - 23), ("one outside the window", 199 - 24), ("page border", 192),
+                                       ("itself only", None))),
+                         ("biased", (("far back", 7), ("a page border far back", 16), ("near", 190), ("itself only", None)))):
+        cfg, weights = _hand_made(kind)
+        engine, _ = _engine(tmp_path / kind, cfg, 31, "fp32", weights=weights)
+        seen = {}
+        for where, at in places:
+            ids = list(base)
+            if at is not None:
+                ids[at] = 2
+            ids[199] = 1
+            requests = {"r": ids}
+            ref = _reference(cfg, weights, requests)
+            for steps in (replay.whole(requests), replay.tail_one_by_one(requests, tail=3), replay.portions(requests, sizes=(64, 2, 33))):
+                got = replay.run_trace(engine, engine.new_cache(14, 16, 1), steps)
+                assert _worst(got, ref) < F32_TOL, where
+            seen[where] = ref["r"][199]
+        moved = lambda a, b: float(np.sqrt(np.mean((seen[a] - seen[b]) ** 2)) / np.sqrt(np.mean(seen[b] ** 2)))
+        if kind == "windowed":
+            assert moved("window edge", "itself only") > 0.1 and moved("page border", "itself only") > 0.1
+            assert moved("one outside the window", "itself only") < 1e-6
+        else:
+            assert min(moved("far back", "itself only"), moved("a page border far back", "itself only"), moved("near", "itself only")) > 0.1
+
+
+def test_a_sink_that_takes_nearly_everything(tmp_path):
+    """Sinks far above and far below the scores: the heads' results all but vanish, or the sink does."""
+    cfg = zm.config([zm.windowed(window=7, mlp=None)])
+    for value in (25.0, -25.0):
+        weights = zm.make_weights(cfg, 8, torch.float32)
+        weights["l0.mix.sink"] = torch.full((6,), value)
+        weights["l0.mix.sink"][2] = 0.3
+        engine, _ = _engine(tmp_path / str(value), cfg, 8, "fp32", weights=weights)
+        requests = {"r": _tokens(30, cfg["vocab"], 3)}
+        ref = _reference(cfg, weights, requests)
+        for steps in (replay.whole(requests), replay.tail_one_by_one(requests, tail=20)):
+            assert _worst(replay.run_trace(engine, engine.new_cache(4, 16, 1), steps), ref) < F32_TOL
+
+
+def test_long_decoding_through_recorded_steps(tmp_path):
+    """300 tokens one by one after a short prompt: windows pass over decoded tokens many times, pages of the sliding
+    layers are given back and used again, the temperature steps, the memory is carried, and the recorded step is replayed."""
+    cfg = zm.MIXED
+    engine, weights = _engine(tmp_path, cfg, 14, "fp32")
+    ids = _tokens(310, cfg["vocab"], 4)
+    ref = _reference(cfg, weights, {"r": ids})
+    steps = replay.tail_one_by_one({"r": ids}, tail=300)
+    got = replay.run_trace(engine, engine.new_cache(20, 16, 2), steps)
+    assert _covered(got, {"r": ids}) and _worst(got, ref) < F32_TOL
+    assert engine.runner.graph_replays >= 299
+
+
+def test_long_decoding_in_bfloat16_on_the_matrix_cores(tmp_path):
+    cfg = zm.ALIGNED
+    engine, weights = _engine(tmp_path, cfg, 18, "bf16")
+    ids = _tokens(200, cfg["vocab"], 4)
+    whole = _stacked(replay.run_trace(engine, engine.new_cache(16, 16, 1), replay.whole({"r": ids})))
+    got = replay.run_trace(engine, engine.new_cache(16, 16, 2), replay.tail_one_by_one({"r": ids}, tail=190))
+    assert _mean(got, whole) < BF16_BETWEEN_SCHEDULES / 2 and _most(got, whole) < BF16_BETWEEN_SCHEDULES
+    assert engine.runner.graph_replays >= 189
+
+
+def test_first_tokens_of_a_sequence(tmp_path):
+    cfg = zm.MIXED
+    engine, weights = _engine(tmp_path, cfg, 15, "fp32")
+    requests = {f"n{n}": _tokens(n, cfg["vocab"], 30 + n) for n in range(1, 7)}
+    ref = _reference(cfg, weights, requests)
+    for steps in (replay.whole(requests), replay.tail_one_by_one(requests, tail=8), replay.mixed(requests, max_live=4, seed=3)):
+        got = replay.run_trace(engine, engine.new_cache(8, 16, 4), steps)
+        assert _worst(got, ref) < F32_TOL
+
+
+def test_greedy_generation_through_the_entry_point_and_the_scheduler(tmp_path):
+    cfg = zm.MIXED
+    engine, weights = _engine(tmp_path, cfg, 16, "fp32")
+    prompts = [_tokens(9, cfg["vocab"], 1), _tokens(30, cfg["vocab"], 2), _tokens(1, cfg["vocab"], 3)]
+    new = 12
+    w = {k: v.float() for k, v in weights.items()}
+
+    def plain_greedy(ids):
+        ids = list(ids)
+        for _ in range(new):
+            ids.append(int(plain.forward(cfg, w, ids)[-1].argmax()))
+        return ids
+
+    want = [plain_greedy(p) for p in prompts]
+    for p, out_want in zip(prompts, want):
+        out, finish = engine.generate(p, new)
+        assert out == out_want and finish == "length"
+    from llmengine import BlockManager, ContinuousBatchScheduler
+    sched = ContinuousBatchScheduler(engine, BlockManager(num_blocks=12, block_size=16), max_concurrent=2,
+                                     max_prefill_tokens_per_step=16)
+    for p in prompts:
+        sched.enqueue(p, new)
+    sched.run_until_idle()
+    assert [r.token_ids for r in sched.results] == want
+
+
+def test_the_trace_runner_replays_a_model_of_this_design(tmp_path):
+    import json
+    import os
+    import subprocess
+    import sys
+    cfg = zm.MIXED
+    folder, weights = zm.write_model(tmp_path / "model", cfg, 17, torch.float32)
+    requests = {"a": _tokens(40, cfg["vocab"], 1), "b": _tokens(21, cfg["vocab"], 2)}
+    steps = replay.mixed(requests, max_live=2, seed=5)
+    ref = _reference(cfg, weights, requests)
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", str(replay.trace_peak_tokens(steps))],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+    done = {rid: 0 for rid in requests}
+    for s in steps:
+        rows = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(-1, cfg["vocab"])
+        r = 0
+        for e in s["entries"]:
+            for w in e["want"]:
+                want = ref[e["id"]][done[e["id"]] + w]
+                assert np.sqrt(np.mean((rows[r] - want) ** 2)) / np.sqrt(np.mean(want ** 2)) < F32_TOL
+                r += 1
+            done[e["id"]] += len(e["tokens"])
+
+
+def test_the_command_line_generates_with_random_weights_of_this_design(tmp_path):
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfgf = tmp_path / "cfg.json"
+    cfgf.write_text(json.dumps(zm.ALIGNED))
+    pf = tmp_path / "prompts.txt"
+    pf.write_text("1 2 3\n7,8,9,10,11\n")
+    out = subprocess.run([sys.executable, os.path.join(root, "bin", "llmengine-cli"), "--random", str(cfgf), "--seed", "3",
+                          "--prompt-file", str(pf), "--max-new-tokens", "4", "--temperature", "0.7"],
+                         capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    recs = [json.loads(line) for line in out.stdout.strip().splitlines()]
+    assert [len(r["token_ids"]) for r in recs] == [7, 9] and all(r["finish_reason"] == "length" for r in recs)
