@@ -20,7 +20,10 @@ measurements at further sizes and context lengths; the default run is the 1B sha
 a residual in several streams) beside Llama with layers of the same sizes: prefill and decode of both;
 `--design bidirax` the Bidirax design instead (latent attention, rotated and windowed, dense and expert feed-forwards),
 `--design zetonex` the Zetonex design (windowed attention with two score maps or with keys as values, dense feed-forwards
-with biases and clamped experts chosen by a table, a stretch of layers that runs two passes).
+with biases and clamped experts chosen by a table, a stretch of layers that runs two passes),
+`--design zapolorn` the Zapolorn design (sublayers normed behind; windowed attention with sinks and head gates, one layer in
+three reading the keys of the layer in front; attention with a bias by distance beside a gated linear attention; dense
+feed-forwards and experts that weigh their input).
 
 `--phase mixed` times one step of continuous batching (a prompt portion beside decoded tokens of
 other requests), `--phase portion` portions of one long prompt. `--phase serve` is another workload (with `--shape 3b`: 32 requests with prompts of 64 to 3,072
@@ -141,6 +144,33 @@ def zetonex_at(width: int, ff: int, heads: int, layers: int, vocab: int, only: s
     return out
 
 
+def zapolorn_at(width: int, ff: int, heads: int, layers: int, vocab: int, only: str = "") -> dict:
+    """Zapolorn layers of a Llama layer's width, heads and active feed-forward size: windowed attention (heads of 64, a quarter
+    as many key heads, a window of 1,024, a sink and a gate per head) with a dense feed-forward; the pair of mixers (attention
+    over everything before with a bias by distance, and a gated linear attention of half the heads with keys of 64 over values
+    of 128) with 16 experts (2 a token, a quarter of the feed-forward size each, beside a shared one of half of it); then a
+    windowed attention that reads the keys and values of the first, with the same experts."""
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": ff // 4}, "shared": {"ff": ff // 2}}
+    win = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 1024},
+           "rot": {"base": 250000.0, "dims": 64, "scaling": {"factor": 8.0}}}
+    par = {"left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125,
+                    "q_temp": {"coef": 0.5, "every": 1024}},
+           "right": {"heads": max(1, heads // 2), "dim": 64, "vdim": 128, "tau": 16.0, "rank": 64},
+           "left_scale": 0.8, "right_scale": 1.1}
+    out = []
+    for i in range(layers):
+        kind = only or ("windowed", "parallel", "windowed_shared")[i % 3]
+        if kind == "parallel":
+            out.append({"type": "parallel", "mixer": par, "mlp": moe})
+        elif kind == "windowed_shared" and i >= 2 and "kv_from" not in out[i - 2]["mixer"] and out[i - 2]["type"] == "attention":
+            out.append({"type": "attention", "mixer": dict(win, kv_from=i - 2), "mlp": moe})
+        else:
+            out.append({"type": "attention", "mixer": win, "mlp": dense})
+    return {"architecture": "Zapolorn", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6},
+            "logit_scale": 1.0, "layers": out}
+
+
 def design(args) -> int:
     """Prefill (one prompt of --prefill-tokens) and decode (--batch requests at --context) of the Rilonex design and of
     Llama with layers of the same width, feed-forward size and number of heads: tokens/s of both and their ratio, per
@@ -155,6 +185,7 @@ def design(args) -> int:
         row = {"size": size, "width": width, "ff": ff, "heads": heads, "layers": layers}
         other = (bidirax_at(width, ff, heads, layers, vocab, only=args.design_only) if args.design == "bidirax"
                  else zetonex_at(width, ff, heads, layers, vocab, only=args.design_only) if args.design == "zetonex"
+                 else zapolorn_at(width, ff, heads, layers, vocab, only=args.design_only) if args.design == "zapolorn"
                  else rilonex_at(width, ff, heads, layers, vocab, only=args.design_only))
         for name, cfg in (("llama", llama_at(width, ff, heads, layers, vocab)), (args.design, other)):
             if args.design_skip_llama and name == "llama":
@@ -398,10 +429,11 @@ def main() -> int:
                          "steps of --portion prompt tokens of one request behind --context tokens; 'mixed': such a "
                          "portion beside one decoded token of --batch other requests")
     ap.add_argument("--design-sizes", default="1k,2k", help="design: sizes to run, of " + ",".join(sorted(DESIGN_SIZES)))
-    ap.add_argument("--design", default="rilonex", choices=["rilonex", "bidirax", "zetonex"], help="design: which design runs beside Llama")
+    ap.add_argument("--design", default="rilonex", choices=["rilonex", "bidirax", "zetonex", "zapolorn"],
+                    help="design: which design runs beside Llama")
     ap.add_argument("--design-only", default="", choices=["", "rglru", "channel_delta", "parallel", "rotated", "windowed", "differential", "gated"],
                     help="design: a model of this kind of layer only (the first three Rilonex, the next two Bidirax, the last "
-                         "two Zetonex)")
+                         "two Zetonex; Zapolorn: windowed or parallel)")
     ap.add_argument("--design-skip-llama", action="store_true", help="design: time the design alone")
     ap.add_argument("--portion", type=int, default=256, help="portion: prompt tokens a step")
     ap.add_argument("--decode-len", type=int, default=700, help="mixed: tokens of the shortest decoding request "

@@ -65,11 +65,20 @@ template <int MODE> __device__ __forceinline__ float gate_act(float g) {
 }
 // What kGatedExtraBF16 does around the activation. bias [N] in the order of w's rows (so in the order of the product's
 // columns): added to gate and up first. limit > 0: gate <- min(gate, limit), up <- clamp(up, -limit, limit) and the
-// value is gate sigmoid(alpha gate) (up + 1); otherwise silu(gate) up.
+// value is gate sigmoid(alpha gate) (up + 1); otherwise silu(gate) up. pair_scale with row_pair: the gate and up sums of
+// row m are multiplied by pair_scale[row_pair[m]] first (0 where row_pair[m] < 0), which is the layer run on that multiple
+// of its input (an expert whose weight is on its input).
 struct GateExtra {
     const bf16* bias = nullptr;
     float limit = 0.f, alpha = 1.f;
+    const int* row_pair = nullptr;
+    const float* pair_scale = nullptr;
 };
+__device__ __forceinline__ float gate_row_scale(const GateExtra& gx, int m) {
+    if (gx.pair_scale == nullptr) return 1.f;
+    const int pair = gx.row_pair[m];
+    return pair < 0 ? 0.f : gx.pair_scale[pair];
+}
 // bg, bu: the biases of this gate and up value (zero where there are none).
 template <int MODE> __device__ __forceinline__ float gated_value(float g, float u, const GateExtra& gx, float bg, float bu) {
     if (MODE != kGatedExtraBF16) return gate_act<MODE>(g) * u;
@@ -297,9 +306,10 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
                     bgv = *reinterpret_cast<const bf16x8*>(gx.bias + n);
                     buv = *reinterpret_cast<const bf16x8*>(gx.bias + n + 16);
                 }
+                const float rs = MODE == kGatedExtraBF16 ? gate_row_scale(gx, m) : 1.f;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    const float gt = gp[e], up = gp[16 + e];
+                    const float gt = gp[e] * rs, up = gp[16 + e] * rs;
                     o[e] = static_cast<__bf16>(gated_value<MODE>(gt, up, gx, static_cast<float>(bgv[e]), static_cast<float>(buv[e])));
                 }
                 const int unit = (n0 + (piece / 2) * 32) / 2 + (piece % 2) * 8;
@@ -364,7 +374,8 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
                 for (int j = 0; j + 1 < WNT; j += 2) {
                     const int unit = (n0 + wn + j * 16) / 2 + r;        // tile column pair (gate, up)
                     if (2 * unit >= N) continue;
-                    const float gt = acc[i][j][e], up = acc[i][j + 1][e];
+                    const float rs = MODE == kGatedExtraBF16 ? gate_row_scale(gx, m) : 1.f;
+                    const float gt = acc[i][j][e] * rs, up = acc[i][j + 1][e] * rs;
                     float bg = 0.f, bu = 0.f;
                     if (MODE == kGatedExtraBF16 && gx.bias != nullptr) {
                         bg = static_cast<float>(gx.bias[n0 + wn + j * 16 + r]);
@@ -1254,14 +1265,19 @@ extern "C" int llme_gemm_bf16_gated_extra(const void* a, const void* w, void* ou
     return rc;
 }
 
-// The experts' gate/up product (llme_gemm_bf16_grouped with tile_group given) with the clamped swish; experts have no biases.
+// The experts' gate/up product (llme_gemm_bf16_grouped with tile_group given) with the clamped swish (limit > 0) or SiLU;
+// experts have no biases. pair_scale (or null): a place's sums are multiplied by pair_scale[row_index[place]] in front of
+// the activation (experts that weigh their input).
 extern "C" int llme_gemm_bf16_grouped_gated_extra(const void* a, const void* w, void* out, int N, int K, int tile, int max_tiles,
                                                   const int* tile_group, const int* n_tiles, const int* row_index, int gather_div,
-                                                  long a_rows, int groups, float limit, float alpha, hipStream_t stream) {
-    if (limit < 0.f || tile_group == nullptr) return kErrBadArgument;
+                                                  long a_rows, int groups, float limit, float alpha, const float* pair_scale,
+                                                  hipStream_t stream) {
+    if (limit < 0.f || tile_group == nullptr || (pair_scale != nullptr && row_index == nullptr)) return kErrBadArgument;
     t_gate_extra.bias = nullptr;
     t_gate_extra.limit = limit;
     t_gate_extra.alpha = alpha;
+    t_gate_extra.row_pair = pair_scale != nullptr ? row_index : nullptr;
+    t_gate_extra.pair_scale = pair_scale;
     const int rc = llme_gemm_bf16_grouped(a, w, out, kBF16, 4, N, K, tile, max_tiles, tile_group, n_tiles, row_index, gather_div,
                                           a_rows, groups, 0, stream);
     t_gate_extra = GateExtra{};

@@ -327,27 +327,31 @@ def moe_gemm(a: torch.Tensor, w: torch.Tensor, gated: bool, group: int, out: tor
                                  int(group), GATE_ACTIVATIONS[activation], stream()), "moe_gemm")
 
 
-declare("llme_gemm_bf16_grouped_gated_extra", [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _i, ctypes.c_long, _i, _f, _f, _vp])
+declare("llme_gemm_bf16_grouped_gated_extra", [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _i, ctypes.c_long, _i, _f, _f, _vp, _vp])
 
 
 def moe_gemm_clamped(a: torch.Tensor, w: torch.Tensor, group: int, out: torch.Tensor, place_pair: torch.Tensor,
                      tile_expert: torch.Tensor, n_tiles: torch.Tensor, tile: int, gather_div: int, limit: float, alpha: float,
-                     choices=None) -> bool:
+                     choices=None, pair_scale: torch.Tensor | None = None) -> bool:
     """The experts' gate/up product with the clamped swish in the tile kernel's epilogue, where that fits (returns False
     where not): per place, g = min(gate a, limit), u = clamp(up a, -limit, limit), out[place] = g sigmoid(alpha g) (u + 1);
-    w [experts, 2 N, K] with gate and up rows in alternating groups of 16."""
+    w [experts, 2 N, K] with gate and up rows in alternating groups of 16. pair_scale [pairs] (32-bit): a place's two sums
+    are first multiplied by its pair's entry (an expert that runs on its weight times the input); with limit 0 the
+    activation is then SiLU."""
     require(w, "w", _FLOATS, (None, None, None))
     E, rows_w, K = w.shape
     if not (tile in MOE_FAST_TILES and _grouped_fits(a, w, choices) and group == 16 and out.dtype == torch.bfloat16
-            and rows_w % 32 == 0 and gather_div > 0 and limit > 0):
+            and rows_w % 32 == 0 and gather_div > 0 and (limit > 0 or (limit == 0 and pair_scale is not None))):
         return False
+    if pair_scale is not None:
+        require(pair_scale, "pair_scale", torch.float32, (None,))
     require(a, "a", torch.bfloat16, (None, K))
     cap = place_pair.shape[0]
     require(out, "out", torch.bfloat16, (cap, rows_w // 2))
     require(tile_expert, "tile_expert", torch.int32, (cap // tile,))
     check(entry("llme_gemm_bf16_grouped_gated_extra")(ptr(a), ptr(w), ptr(out), rows_w, K, tile, cap // tile, ptr(tile_expert),
                                                       ptr(n_tiles), ptr(place_pair), int(gather_div), a.shape[0], E, float(limit),
-                                                      float(alpha), stream()), "moe_gemm_clamped")
+                                                      float(alpha), ptr(pair_scale), stream()), "moe_gemm_clamped")
     return True
 
 

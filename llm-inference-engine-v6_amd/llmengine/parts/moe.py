@@ -116,6 +116,10 @@ class MixtureOfExperts(FeedForward):
                                                                              tile_expert, n_tiles, tile, top, self.limit, 1.702,
                                                                              step.choices):
             pass                            # (clamps and activation in the product's epilogue)
+        elif self.weight_on == "input" and self.activation == "silu" and ops.latent.moe_gemm_clamped(
+                x, self.w_gate_up, self.group, act, place_pair, tile_expert, n_tiles, tile, top, 0.0, 1.0, step.choices,
+                pair_scale=wts.view(-1)):
+            pass                            # (a place's sums times its pair's weight, then the activation, in the product's epilogue)
         elif self.weight_on == "input":
             # the gate and up sums as 32-bit rows, each row times its pair's weight, then the activation, in one pass
             gu = step.buffer("moe.gate_up", (cap, 2 * FF), f32)
