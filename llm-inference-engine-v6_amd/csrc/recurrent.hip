@@ -307,14 +307,32 @@ __global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restric
 }
 
 // decay[t, e] = sigmoid(z[t, e] + bias[e])^(1 / tau) = exp(-softplus(-(z + bias)) / tau): a decay per channel from a
-// logit, flattened by a temperature. z is a column range of a 32-bit buffer; bias (null: none) in its stored type.
+// logit, flattened by a temperature. z is a column range of a 32-bit buffer, or, where a2 [n, rank] is given, made here
+// from the first stage of a two-stage map: z[t, e] = sum_r a2[e, r] low[t, r] (32-bit sums). bias (null: none) and a2
+// in their stored type.
 template <typename TW>
-__global__ __launch_bounds__(256) void sigmoid_decay_kernel(const float* __restrict__ z, int ld, const TW* __restrict__ bias,
-                                                            float inv_tau, float* __restrict__ decay, int n) {
+__global__ __launch_bounds__(256) void sigmoid_decay_kernel(const float* __restrict__ z, int ld, const TW* __restrict__ a2, int rank,
+                                                            const TW* __restrict__ bias, float inv_tau, float* __restrict__ decay,
+                                                            int n) {
     const int t = blockIdx.y;
     const int e = blockIdx.x * 256 + threadIdx.x;
     if (e >= n) return;
-    const float x = z[static_cast<size_t>(t) * ld + e] + (bias != nullptr ? to_float(bias[e]) : 0.f);
+    const float* zr = z + static_cast<size_t>(t) * ld;
+    float x;
+    if (a2 != nullptr) {
+        const TW* row = a2 + static_cast<size_t>(e) * rank;
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        int r = 0;
+        for (; r + 4 <= rank; r += 4) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = fmaf(to_float(row[r + i]), zr[r + i], acc[i]);
+        }
+        for (; r < rank; ++r) acc[0] = fmaf(to_float(row[r]), zr[r], acc[0]);
+        x = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+    } else {
+        x = zr[e];
+    }
+    if (bias != nullptr) x += to_float(bias[e]);
     decay[static_cast<size_t>(t) * n + e] = expf(-softplusf_(-x) * inv_tau);
 }
 
@@ -344,12 +362,23 @@ __device__ __forceinline__ float sum_of_lanes(float v) {
 // DELTA false is the plain linear rule (gated linear attention): nothing is read back before the write,
 //   M <- g * M;  M <- M + k v^T;  o = M^T q,
 // and beta is not looked at. Every read is multiplied by o_scale (a scale on the queries).
+//
+// The linear rule with a decay per channel is linear in M with a diagonal map, so long runs of rows can be cut into
+// chunks of `chunk` rows that are walked side by side (grid z = request x chunk), in three launches:
+//   phase 1: every chunk from an empty memory, no reads: what the chunk adds (B, into chunk_state) and the product
+//            of its decays (P, into chunk_decay);
+//   carry  : per request, chunk by chunk, M_start(c) = M; M <- P(c) M + B(c); chunk_state then holds M_start, the slot
+//            the memory behind the last row;
+//   phase 3: every chunk again from its M_start, with the reads.
+// phase 0 is the walk over all rows of a request in one go.
 template <int R, int LPC, bool PER_CHANNEL, bool DELTA>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ qkv, int ld, int q_col, int k_col, int v_col,
                                                          const float* __restrict__ beta, const float* __restrict__ decay,
                                                          float* __restrict__ state, const int* __restrict__ q_start,
  const int* __restrict__ slots, float* __restrict__ o, int heads,
-                                                         int kv_heads, int dim, int vdim, float o_scale) {
+                                                         int kv_heads, int dim, int vdim, float o_scale, int phase, int chunk,
+                                                         int n_chunks, float* __restrict__ chunk_state,
+                                                         float* __restrict__ chunk_decay) {
     constexpr int DP = LPC * R;                             // a row's k (q, decay) padded with zeros to this many
     constexpr int kDeltaCols = 256 / LPC;                   // columns of the state a workgroup owns
     constexpr int NV = PER_CHANNEL ? 3 : 2;
@@ -358,19 +387,27 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
     constexpr int NF = (BLOCK + 255) / 256;
     static_assert(NF <= kDeltaFetch, "a block of rows is more than the threads fetch");
     __shared__ float lds[2 * BLOCK];
-    const int s = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * kDeltaCols;
+    const int s = phase == 0 ? blockIdx.z : blockIdx.z / n_chunks, h = blockIdx.y, col0 = blockIdx.x * kDeltaCols;
     const int tid = threadIdx.x;
     const int cl = tid / LPC, l = tid % LPC;
     const int col = col0 + cl;
     const bool live = col < vdim;
     const int kvh = h / (heads / kv_heads);
-    const int first = q_start[s], last = q_start[s + 1];
-    float* M = state + ((static_cast<size_t>(slots[s]) * heads + h) * vdim + (live ? col : 0)) * dim;
-    float m[R];
+    int first = q_start[s], last = q_start[s + 1];
+    if (phase != 0) {
+        first += (blockIdx.z % n_chunks) * chunk;
+        if (first >= last) return;                          // (the request has fewer chunks than the longest one)
+        last = first + chunk < last ? first + chunk : last;
+    }
+    // where the memory comes from and where it goes: the request's slot, or this chunk's place in chunk_state
+    float* M = phase == 0 ? state + ((static_cast<size_t>(slots[s]) * heads + h) * vdim + (live ? col : 0)) * dim
+                          : chunk_state + ((static_cast<size_t>(blockIdx.z) * heads + h) * vdim + (live ? col : 0)) * dim;
+    float m[R], pp[R];
 #pragma unroll
     for (int i = 0; i < R; ++i) {
         const int d = l * R + i;
-        m[i] = (live && d < dim) ? M[d] : 0.f;
+        m[i] = (live && d < dim && phase != 1) ? M[d] : 0.f;
+        pp[i] = 1.f;
     }
     const int n_dec = PER_CHANNEL ? heads * dim : heads;
     // Where each of a thread's NF values of a block of rows comes from is the same for every block: the address for the
@@ -466,6 +503,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
 #pragma unroll
             for (int i = 0; i < R; ++i) {
                 m[i] *= PER_CHANNEL ? gg[i] : g_head;
+                if (PER_CHANNEL && !DELTA) pp[i] *= gg[i];
                 dots[i % 2] += m[i] * kk[i];
             }
             const float w = DELTA ? bt * (vv - sum_of_lanes<LPC>(dots[0] + dots[1])) : vv;
@@ -476,7 +514,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
                 reads[i % 2] += m[i] * qq[i];
             }
             const float read = sum_of_lanes<LPC>(reads[0] + reads[1]);
-            if (live && l == 0) o[static_cast<size_t>(t0 + tt) * heads * vdim + h * vdim + col] = read * o_scale;
+            if (live && l == 0 && phase != 1) o[static_cast<size_t>(t0 + tt) * heads * vdim + h * vdim + col] = read * o_scale;
         };
         if (nt == kDeltaRows) {             // a whole block: no test between its rows, so that the rows' loads from LDS run ahead
 #pragma unroll
@@ -490,11 +528,39 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
             cur ^= 1;
         }
     }
+    if (phase == 3) return;
 #pragma unroll
     for (int i = 0; i < R; ++i) {
         const int d = l * R + i;
         if (live && d < dim) M[d] = m[i];
+        if (PER_CHANNEL && !DELTA && phase == 1 && col == 0 && d < dim)
+            chunk_decay[(static_cast<size_t>(blockIdx.z) * heads + h) * dim + d] = pp[i];
     }
+}
+
+// The carry between the chunks of the linear rule: one thread per (request, head, column, key channel).
+__global__ __launch_bounds__(256) void linear_rule_carry_kernel(float* __restrict__ state, const int* __restrict__ q_start,
+                                                                const int* __restrict__ slots, float* __restrict__ chunk_state,
+                                                                const float* __restrict__ chunk_decay, int heads, int dim, int vdim,
+                                                                int chunk, int n_chunks) {
+    const int s = blockIdx.y;
+    const size_t per = static_cast<size_t>(heads) * vdim * dim;
+    const size_t e = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (e >= per) return;
+    const int d = static_cast<int>(e % dim);
+    const int h = static_cast<int>(e / (static_cast<size_t>(vdim) * dim));
+    const int rows = q_start[s + 1] - q_start[s];
+    const int nc = (rows + chunk - 1) / chunk;
+    float* slot = state + static_cast<size_t>(slots[s]) * per + e;
+    float m = *slot;
+    for (int c = 0; c < nc; ++c) {
+        const size_t z = static_cast<size_t>(s) * n_chunks + c;
+        float* at = chunk_state + z * per + e;
+        const float add = *at;
+        *at = m;
+        m = fmaf(chunk_decay[(z * heads + h) * dim + d], m, add);
+    }
+    if (nc > 0) *slot = m;
 }
 
 // out[t, h, j] = scale * o[t, h, j] / sqrt(mean_j o^2 + eps) * w[j] * gate, in the activation type.
@@ -664,24 +730,40 @@ extern "C" int llme_delta_gates(const void* b_in, int ld_b, const void* a_in, in
     return launch_status();
 }
 
-extern "C" int llme_sigmoid_decay(const void* z, int ld, const void* bias, int w_dtype, float tau, void* decay, int T, int n,
-                                  hipStream_t stream) {
+extern "C" int llme_sigmoid_decay(const void* z, int ld, const void* a2, int rank, const void* bias, int w_dtype, float tau,
+                                  void* decay, int T, int n, hipStream_t stream) {
     if (T <= 0 || n <= 0) return 0;
-    if (!(tau > 0.f) || ld < n) return kErrBadArgument;
+    if (!(tau > 0.f) || ld < (a2 != nullptr ? rank : n) || (a2 != nullptr && rank <= 0)) return kErrBadArgument;
     const dim3 grid((n + 255) / 256, T);
-    LLME_BY_W(w_dtype, (sigmoid_decay_kernel<TW><<<grid, 256, 0, stream>>>(static_cast<const float*>(z), ld, static_cast<const TW*>(bias),
-                                                                       1.0f / tau, static_cast<float*>(decay), n)));
+    LLME_BY_W(w_dtype, (sigmoid_decay_kernel<TW><<<grid, 256, 0, stream>>>(static_cast<const float*>(z), ld, static_cast<const TW*>(a2),
+                                                                       rank, static_cast<const TW*>(bias), 1.0f / tau,
+                                                                       static_cast<float*>(decay), n)));
     return launch_status();
 }
 
 template <int R, int LPC>
 static void launch_delta_rule(bool per_channel, int n_seq, hipStream_t stream, const float* qkv, int ld, int q_col, int k_col,
                               int v_col, const float* beta, const float* decay, float* state, const int* q_start,
-                              const int* slots, float* o, int heads, int kv_heads, int dim, int vdim, float o_scale) {
+                              const int* slots, float* o, int heads, int kv_heads, int dim, int vdim, float o_scale, int chunk,
+                              int n_chunks, float* chunk_state, float* chunk_decay) {
     const dim3 grid((vdim + 256 / LPC - 1) / (256 / LPC), heads, n_seq);
 #define LLME_DR(PC, DL)                                                                                                          \
     delta_rule_kernel<R, LPC, PC, DL><<<grid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots, o, \
-                                                                 heads, kv_heads, dim, vdim, o_scale)
+                                                                 heads, kv_heads, dim, vdim, o_scale, 0, 0, 1, nullptr, nullptr)
+    if (chunk > 0) {
+        // (the linear rule with a decay per channel, in chunks walked side by side)
+        const dim3 cgrid(grid.x, heads, n_seq * n_chunks);
+        const size_t per = static_cast<size_t>(heads) * vdim * dim;
+        delta_rule_kernel<R, LPC, true, false><<<cgrid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots,
+                                                                         o, heads, kv_heads, dim, vdim, o_scale, 1, chunk, n_chunks,
+                                                                         chunk_state, chunk_decay);
+        linear_rule_carry_kernel<<<dim3(static_cast<unsigned>((per + 255) / 256), n_seq), 256, 0, stream>>>(
+            state, q_start, slots, chunk_state, chunk_decay, heads, dim, vdim, chunk, n_chunks);
+        delta_rule_kernel<R, LPC, true, false><<<cgrid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots,
+                                                                         o, heads, kv_heads, dim, vdim, o_scale, 3, chunk, n_chunks,
+                                                                         chunk_state, chunk_decay);
+        return;
+    }
     if (beta != nullptr) {
         if (per_channel) LLME_DR(true, true);
         else LLME_DR(false, true);
@@ -694,18 +776,25 @@ static void launch_delta_rule(bool per_channel, int n_seq, hipStream_t stream, c
 
 // qkv [T, ld] 32-bit with unit q at q_col, unit k at k_col (kv_heads x dim each) and v at v_col (heads x vdim);
 // beta [T, heads], or null for the linear rule; decay [T, heads, dim] or [T, heads]; state [slots, heads, vdim, dim];
-// o [T, heads, vdim] 32-bit, times o_scale.
+// o [T, heads, vdim] 32-bit, times o_scale. chunk > 0 (the linear rule with a decay per channel only): every request's
+// rows in chunks of that many, walked side by side; n_chunks = the most chunks a request has; chunk_state
+// [n_seq * n_chunks, heads, vdim, dim] and chunk_decay [n_seq * n_chunks, heads, dim] are scratch.
 extern "C" int llme_delta_rule(const void* qkv, int ld, int q_col, int k_col, int v_col, const void* beta, const void* decay,
                                int per_channel, void* state, const void* q_start, const void* slots, void* o, int n_seq,
-                               int heads, int kv_heads, int dim, int vdim, float o_scale, hipStream_t stream) {
+                               int heads, int kv_heads, int dim, int vdim, float o_scale, int chunk, int n_chunks,
+                               void* chunk_state, void* chunk_decay, hipStream_t stream) {
     if (n_seq <= 0 || heads <= 0) return 0;
     if (kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return kErrBadArgument;
     if (dim > 256) return kErrUnsupported;
+    if (chunk < 0 || (chunk > 0 && (beta != nullptr || !per_channel || n_chunks <= 0 || chunk_state == nullptr ||
+                                    chunk_decay == nullptr || static_cast<long>(n_seq) * n_chunks > 65535)))
+        return kErrBadArgument;
 #define LLME_DELTA(R_, L_)                                                                                               \
     launch_delta_rule<R_, L_>(per_channel != 0, n_seq, stream, static_cast<const float*>(qkv), ld, q_col, k_col, v_col, \
                           static_cast<const float*>(beta), static_cast<const float*>(decay), static_cast<float*>(state), \
                           static_cast<const int*>(q_start), static_cast<const int*>(slots), static_cast<float*>(o), heads, \
-                          kv_heads, dim, vdim, o_scale)
+                          kv_heads, dim, vdim, o_scale, chunk, n_chunks, static_cast<float*>(chunk_state),                 \
+                          static_cast<float*>(chunk_decay))
     if (dim <= 16) LLME_DELTA(2, 8);
     else if (dim <= 32) LLME_DELTA(4, 8);
     else if (dim <= 64) LLME_DELTA(4, 16);

@@ -34,8 +34,11 @@ declare("llme_rglru_scan_chunked", [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, 
 declare("llme_copy_cols", [_vp, _i, _vp, _i, _i, _i, _vp])
 declare("llme_unit_heads", [_vp, _i, _i, _i, _i, _i, _f, _f, _f, _vp])
 declare("llme_delta_gates", [_vp, _i, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp])
-declare("llme_delta_rule", [_vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp])
-declare("llme_sigmoid_decay", [_vp, _i, _vp, _i, _f, _vp, _i, _i, _vp])
+declare("llme_delta_rule", [_vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _vp, _vp, _vp])
+LINEAR_RULE_CHUNK = 64                  # rows of a chunk where the linear rule's long runs of rows are walked side by side
+LINEAR_RULE_CHUNK_FROM = 192            # the most rows a request brings from which that is done
+LINEAR_RULE_CHUNK_BYTES = 512 << 20     # and the most scratch memory it may take
+declare("llme_sigmoid_decay", [_vp, _i, _vp, _i, _vp, _i, _f, _vp, _i, _i, _vp])
 declare("llme_gated_head_norm", [_vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _f, _f, _vp])
 declare("llme_rotate_write", [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp])
 declare("llme_sigmoid_attention", [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp])
@@ -257,17 +260,26 @@ def delta_gates(b_in: torch.Tensor, a_in: torch.Tensor, a2: torch.Tensor | None,
                                     1 if per_channel else 0, stream()), "delta_gates")
 
 
-def sigmoid_decay(z: torch.Tensor, bias: torch.Tensor | None, tau: float, decay: torch.Tensor) -> None:
-    """decay [T, n] (32-bit) = sigmoid(z + bias)^(1 / tau), z [T, n] a column range of a 32-bit buffer."""
-    T, n = z.shape
-    ld = _cols(z, "z", torch.float32, T, n)
+def sigmoid_decay(z: torch.Tensor, bias: torch.Tensor | None, tau: float, decay: torch.Tensor, a2: torch.Tensor | None = None) -> None:
+    """decay [T, n] (32-bit) = sigmoid(z + bias)^(1 / tau), z [T, n] a column range of a 32-bit buffer; with a2 [n, rank],
+    z [T, rank] is the first stage of a two-stage map and the logit is z a2^T, summed in 32-bit (bias in a2's type)."""
+    T = z.shape[0]
+    n = decay.shape[1] if a2 is not None else z.shape[1]
+    rank = 0
+    if a2 is not None:
+        require(a2, "a2", _FLOATS, (n, None))
+        rank = a2.shape[1]
+        ld = _cols(z, "z", torch.float32, T, rank)
+    else:
+        ld = _cols(z, "z", torch.float32, T, n)
     if bias is not None:
-        require(bias, "bias", _FLOATS, (n,))
+        require(bias, "bias", a2.dtype if a2 is not None else _FLOATS, (n,))
     require(decay, "decay", torch.float32, (T, n))
     if not tau > 0:
         raise KernelError(f"sigmoid_decay: tau={tau} must be > 0")
-    check(entry("llme_sigmoid_decay")(ptr(z), ld, ptr(bias), code(bias.dtype) if bias is not None else 0, float(tau), ptr(decay),
-                                      T, n, stream()), "sigmoid_decay")
+    w_dtype = a2.dtype if a2 is not None else bias.dtype if bias is not None else torch.float32
+    check(entry("llme_sigmoid_decay")(ptr(z), ld, ptr(a2), rank, ptr(bias), code(w_dtype), float(tau), ptr(decay), T, n, stream()),
+          "sigmoid_decay")
 
 
 def delta_rule(qkv: torch.Tensor, beta: torch.Tensor | None, decay: torch.Tensor, state: torch.Tensor, step, o: torch.Tensor,
@@ -276,7 +288,9 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor | None, decay: torch.Tensor
     a column's key channels lie together):
     M <- decay * M; w = beta (v - M^T k); M <- M + k w^T; o = q_scale M^T q. beta None: the linear rule, w = v (nothing
     is read back before the write). qkv [T, (2 kv_heads dim + heads vdim)] holds q, k and v side by side; decay is
-    [T, heads * dim] (per key channel) or [T, heads]."""
+    [T, heads * dim] (per key channel) or [T, heads]. The linear rule with a decay per channel walks long runs of rows
+    (prompts) in chunks side by side: what each chunk adds from an empty memory, the carry from chunk to chunk, then
+    every chunk again from the memory in front of it."""
     T = qkv.shape[0]
     ld = _cols(qkv, "qkv", torch.float32, T, 2 * kv_heads * dim + heads * vdim)
     if heads % kv_heads:
@@ -292,9 +306,19 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor | None, decay: torch.Tensor
     require(o, "o", torch.float32, (T, heads * vdim))
     if T != step.num_tokens:
         raise KernelError("delta_rule: one row per token of the step")
+    chunk, n_chunks, chunk_state, chunk_decay = 0, 0, None, None
+    longest = max(step.new_lens) if step.new_lens else T
+    if beta is None and per_channel and longest >= LINEAR_RULE_CHUNK_FROM:
+        n_chunks = (longest + LINEAR_RULE_CHUNK - 1) // LINEAR_RULE_CHUNK
+        places = step.num_seqs * n_chunks
+        if places <= 65535 and places * heads * vdim * dim * 4 <= LINEAR_RULE_CHUNK_BYTES:
+            chunk = LINEAR_RULE_CHUNK
+            chunk_state = step.buffer("linear_rule.chunk_state", (places, heads, vdim, dim), torch.float32)
+            chunk_decay = step.buffer("linear_rule.chunk_decay", (places, heads, dim), torch.float32)
     check(entry("llme_delta_rule")(ptr(qkv), ld, 0, kv_heads * dim, 2 * kv_heads * dim, ptr(beta), ptr(decay),
                                    1 if per_channel else 0, ptr(state), ptr(step.q_start), ptr(step.slots), ptr(o),
-                                   step.num_seqs, heads, kv_heads, dim, vdim, float(q_scale), stream()), "delta_rule")
+                                   step.num_seqs, heads, kv_heads, dim, vdim, float(q_scale), chunk, n_chunks if chunk else 0,
+                                   ptr(chunk_state), ptr(chunk_decay), stream()), "delta_rule")
 
 
 def gated_head_norm(o: torch.Tensor, weight: torch.Tensor, gate_in: torch.Tensor, g2: torch.Tensor | None, out: torch.Tensor,

@@ -63,7 +63,7 @@ class GatedLinearAttention(ProjectedMixer):
             raise ValueError(f"gated linear attention: a1 {tuple(a1.shape)} and a2 {tuple(a2.shape)} disagree on the rank")
         self.decay_rank = int(a1.shape[0])
         self.a2 = placement.place(a2)
-        self.a2_bias = placement.place(get("a2.b"), f32)
+        self.a2_bias = placement.place(get("a2.b"), self.a2.dtype)
         self.norm_w = placement.place(get("norm"), f32)
 
     def core(self, p, step, cache, o, scale=1.0):
@@ -71,13 +71,9 @@ class GatedLinearAttention(ProjectedMixer):
         heads, dim, vdim = self.heads, self.dim, self.vdim
         C, hv = self.qkv_width, heads * vdim
         g_in = p[:, C:C + hv]
-        # the second stage of the decay's map as a product of its own, its 32-bit input made contiguous first
-        low = step.buffer("linear_attention.decay_low", (T, self.decay_rank), torch.float32)
-        ops.copy_cols(p[:, C + hv:C + hv + self.decay_rank], low)
-        z = step.buffer("linear_attention.decay_in", (T, heads * dim), torch.float32)
-        ops.gemm(low, self.a2, z, choices=step.choices)
+        # the second stage of the decay's map (a 32-bit sum over the rank), its bias and the decay itself in one kernel
         decay = step.buffer("linear_attention.decay", (T, heads * dim), torch.float32)
-        ops.sigmoid_decay(z, self.a2_bias, self.tau, decay)
+        ops.sigmoid_decay(p[:, C + hv:C + hv + self.decay_rank], self.a2_bias, self.tau, decay, a2=self.a2)
         read = step.buffer("linear_attention.read", (T, hv), torch.float32)
         ops.delta_rule(p[:, :C], None, decay, cache.state["memory"], step, read, heads, heads, dim, vdim, per_channel=True,
                        q_scale=float(dim) ** -0.5)

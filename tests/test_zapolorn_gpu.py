@@ -208,6 +208,25 @@ def test_a_slot_that_is_used_again_starts_from_an_empty_memory(tmp_path):
         assert _worst(got, ref) < F32_TOL
 
 
+def test_long_portions_beside_single_tokens_walk_the_memory_in_chunks(tmp_path):
+    """Portions of a few hundred tokens have the linear attention's memory walked in chunks side by side; in the same
+    step other requests bring one token or two, and a request's portion need not end where a chunk ends."""
+    cfg = zm.config([zm.parallel(left_scale=0.3, right_scale=1.5, tau=12.0, mlp=None), zm.parallel(r_heads=3, r_dim=24, r_vdim=5, mlp="dense")])
+    engine, weights = _engine(tmp_path, cfg, 6, "fp32")
+    V = cfg["vocab"]
+    requests = {"long": _tokens(530, V, 1), "other": _tokens(260, V, 2), "short": _tokens(12, V, 3)}
+    ref = _reference(cfg, weights, requests)
+    cut = lambda rid, a, b: {"id": rid, "tokens": requests[rid][a:b], "want": list(range(b - a))}
+    steps = [{"step": 0, "entries": [cut("long", 0, 201), cut("short", 0, 1)], "end": []},
+             {"step": 1, "entries": [cut("short", 1, 3), cut("long", 201, 457), cut("other", 0, 193)], "end": []},
+             {"step": 2, "entries": [cut("other", 193, 260), cut("long", 457, 458), cut("short", 3, 4)], "end": ["other"]},
+             {"step": 3, "entries": [cut("long", 458, 530), cut("short", 4, 12)], "end": ["long", "short"]}]
+    got = replay.run_trace(engine, engine.new_cache(replay.trace_peak_tokens(steps, 16) // 16, 16, 3), steps)
+    assert _covered(got, requests) and _worst(got, ref) < F32_TOL
+    whole = replay.run_trace(engine, engine.new_cache(40, 16, 1), replay.whole(requests))
+    assert _worst(whole, ref) < F32_TOL
+
+
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 def test_far_keys_page_borders_and_window_edges(tmp_path, dtype):
     """Sharp softmaxes over a long prompt: the layers without a window find their keys anywhere among hundreds (the bias by
