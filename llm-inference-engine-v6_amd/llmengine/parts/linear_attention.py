@@ -23,6 +23,8 @@ from .registry import register_part
 
 
 class GatedLinearAttention(ProjectedMixer):
+    FUSED_DECAY_ROWS = 64           # steps of up to this many rows make the decay's logit inside the decay kernel
+
     def __init__(self, hidden_size: int, heads: int, dim: int, vdim: int, tau: float, eps: float, decay_rank: int | None = None):
         if not tau > 0:
             raise ValueError(f"gated linear attention: tau={tau} must be > 0")
@@ -71,9 +73,18 @@ class GatedLinearAttention(ProjectedMixer):
         heads, dim, vdim = self.heads, self.dim, self.vdim
         C, hv = self.qkv_width, heads * vdim
         g_in = p[:, C:C + hv]
-        # the second stage of the decay's map (a 32-bit sum over the rank), its bias and the decay itself in one kernel
         decay = step.buffer("linear_attention.decay", (T, heads * dim), torch.float32)
-        ops.sigmoid_decay(p[:, C + hv:C + hv + self.decay_rank], self.a2_bias, self.tau, decay, a2=self.a2)
+        low_in = p[:, C + hv:C + hv + self.decay_rank]
+        if T <= self.FUSED_DECAY_ROWS:
+            # few rows: the second stage of the decay's map (a 32-bit sum over the rank), its bias and the decay in one kernel
+            ops.sigmoid_decay(low_in, self.a2_bias, self.tau, decay, a2=self.a2)
+        else:
+            # many rows: the second stage as a product of its own, its 32-bit input made contiguous first
+            low = step.buffer("linear_attention.decay_low", (T, self.decay_rank), torch.float32)
+            ops.copy_cols(low_in, low)
+            z = step.buffer("linear_attention.decay_in", (T, heads * dim), torch.float32)
+            ops.gemm(low, self.a2, z, choices=step.choices)
+            ops.sigmoid_decay(z, self.a2_bias, self.tau, decay)
         read = step.buffer("linear_attention.read", (T, hv), torch.float32)
         ops.delta_rule(p[:, :C], None, decay, cache.state["memory"], step, read, heads, heads, dim, vdim, per_channel=True,
                        q_scale=float(dim) ** -0.5)
