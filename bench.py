@@ -153,11 +153,11 @@ def zapolorn_at(width: int, ff: int, heads: int, layers: int, vocab: int, only: 
     dense = {"kind": "dense", "ff": ff}
     moe = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": ff // 4}, "shared": {"ff": ff // 2}}
     win = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 1024},
-           "rot": {"base": 250000.0, "dims": 64, "scaling": {"factor": 8.0}}}
+           "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 4.0}}}
     par = {"left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125,
-                    "q_temp": {"coef": 0.5, "every": 1024}},
-           "right": {"heads": max(1, heads // 2), "dim": 64, "vdim": 128, "tau": 16.0, "rank": 64},
-           "left_scale": 0.8, "right_scale": 1.1}
+                    "q_temp": {"coef": 0.25, "every": 1024}},
+           "right": {"heads": max(1, heads // 2), "dim": 64, "vdim": 128, "tau": 8.0, "rank": 64},
+           "left_scale": 1.0, "right_scale": 1.0}
     out = []
     for i in range(layers):
         kind = only or ("windowed", "parallel", "windowed_shared")[i % 3]

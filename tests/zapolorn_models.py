@@ -70,8 +70,8 @@ ALIGNED = config([parallel(heads=4, kv_heads=2, dim=32, vdim=48, scale=0.1, coef
                            mlp={"kind": "dense", "ff": 128}),
                   windowed(heads=8, kv_heads=2, dim=32, vdim=16, scale=0.2, base=10000.0, dims=16, factor=4.0, window=24, kv_from=1,
                            mlp=feed_forward("moe", ff=32, experts=4, top=1, shared=0)),
-                  parallel(heads=6, kv_heads=1, dim=64, vdim=32, scale=0.09, coef=0.5, every=64, r_heads=2, r_dim=48, r_vdim=32, tau=16.0,
-                           rank=16, left_scale=1.2, right_scale=0.8, mlp={"kind": "dense", "ff": 64})],
+                  parallel(heads=6, kv_heads=1, dim=64, vdim=32, scale=0.09, coef=0.6, every=64, r_heads=2, r_dim=40, r_vdim=24, tau=12.0,
+                           rank=6, left_scale=1.2, right_scale=0.8, mlp={"kind": "dense", "ff": 64})],
                  width=64, vocab=128)
 
 
