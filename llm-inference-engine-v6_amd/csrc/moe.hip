@@ -45,15 +45,20 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
     mx = wave_max(mx);
     float sum = 0.f;
+    if (!sigmoid) {
 #pragma unroll
-    for (int i = 0; i < kMoeMaxPerLane; ++i) {
-        v[i] = sigmoid ? 1.0f / (1.0f + expf(-v[i])) : expf(v[i] - mx);                 // 0 beyond E
-        sum += v[i];
+        for (int i = 0; i < kMoeMaxPerLane; ++i) {
+            v[i] = expf(v[i] - mx);                 // 0 beyond E
+            sum += v[i];
+        }
     }
+    // (sigmoid scores: the experts are chosen by their logits, which order them as the scores do and still tell
+    // experts apart where the 32-bit sigmoid has run into 1 or 0; a chosen expert's score is made from its logit)
     const float inv = sigmoid ? 1.0f : 1.0f / wave_sum(sum);
+    const float none = sigmoid ? -INFINITY : -1.f;
     float chosen_sum = 0.f;
     for (int k = 0; k < top; ++k) {
-        float best = -1.f;
+        float best = none;
         int at = 0x7fffffff;
 #pragma unroll
         for (int i = 0; i < kMoeMaxPerLane; ++i) {
@@ -72,7 +77,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
                 at = oa;
             }
         }
-        const float s = best * inv;
+        const float s = sigmoid ? 1.0f / (1.0f + expf(-best)) : best * inv;
         chosen_sum += s;
         if (lane == 0) {
             ids[static_cast<size_t>(t) * top + k] = at;
@@ -80,7 +85,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
         }
 #pragma unroll
         for (int i = 0; i < kMoeMaxPerLane; ++i)
-            if (lane + i * kWave == at) v[i] = -2.f;        // taken
+            if (lane + i * kWave == at) v[i] = sigmoid ? -INFINITY : -2.f;        // taken
     }
     if (lane == 0) {
         const float f = renorm ? scale / chosen_sum : scale;
