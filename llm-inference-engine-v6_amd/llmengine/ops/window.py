@@ -91,6 +91,7 @@ declare("llme_window_attention_mfma", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _
 WINDOW_MFMA_STAGED = True           # prompts' blocks of keys staged once a workgroup through LDS (False: measurements, tests)
 WINDOW_MFMA_MAX_ENTRIES = 128       # entries of a key or value head that the matrix-core kernel holds
 WINDOW_MFMA_MAX_RUNS = 32
+WINDOW_MFMA_LONG_RUN = 4            # blocks of 32 keys a run from which a step's keys are cut into twice as many runs
 
 
 def window_mfma_fits(k_cache: torch.Tensor, v_cache: torch.Tensor, choices=None) -> bool:
@@ -117,7 +118,11 @@ def window_runs(step, rows_per_token: int, key_heads: int, window: int, keep_fir
         keys = min(keys, window + (16 + rows_per_token - 1) // rows_per_token + min(keep_first, keys))
     tiles = sum((n * rows_per_token + 15) // 16 for n in step.new_lens) * key_heads
     blocks = (keys + 31) // 32 + 1
-    return max_new, max(1, min(WINDOW_MFMA_MAX_RUNS, (4 * mfma.compute_units()) // max(tiles, 1), blocks))
+    runs = max(1, min(WINDOW_MFMA_MAX_RUNS, (4 * mfma.compute_units()) // max(tiles, 1), blocks))
+    if decode and blocks > WINDOW_MFMA_LONG_RUN * runs:
+        # single tokens over long runs (many keys, no window): twice the wavefronts a compute unit, so that a run is half as long
+        runs = max(1, min(WINDOW_MFMA_MAX_RUNS, (8 * mfma.compute_units()) // max(tiles, 1), blocks))
+    return max_new, runs
 
 
 def _fast_window_attention(q, k_cache, v_cache, step, block_table, nq, scale, softcap, window, keep_first, slopes=None):
