@@ -145,6 +145,29 @@ def test_every_schedule_gives_the_plain_logits(tmp_path, cfg_name, dtype):
             assert not cache.manager.live_requests()
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Layers of both kinds in any order with sizes, head counts, windows and constants drawn at random, in 32-bit against
+    the plain model and in bfloat16 from schedule to schedule, with prompts long enough for the memory's chunks."""
+    cfg = zm.random_config(seed)
+    V = cfg["vocab"]
+    requests = {"a": _tokens(300 + 37 * seed, V, seed), "b": _tokens(1 + 11 * seed, V, seed + 50), "c": _tokens(200, V, seed + 90)}
+    schedules = [replay.whole(requests), replay.tail_one_by_one(requests, tail=40 + 20 * seed),
+                 replay.portions(requests, sizes=(64, 2, 33, 200, 7, 1, 129)), replay.mixed(requests, max_live=3, sizes=(50, 3, 24, 2, 210), seed=seed)]
+    weights = zm.make_weights(cfg, seed, torch.float32)
+    engine, _ = _engine(tmp_path / "fp32", cfg, seed, "fp32", weights=weights)
+    ref = _reference(cfg, weights, requests)
+    for steps in schedules:
+        got = replay.run_trace(engine, engine.new_cache(replay.trace_peak_tokens(steps, 16) // 16, 16, 3), steps)
+        assert _covered(got, requests) and _worst(got, ref) < 1.5 * F32_TOL
+    engine, _ = _engine(tmp_path / "bf16", cfg, seed, "bf16")
+    first = None
+    for steps in schedules:
+        got = replay.run_trace(engine, engine.new_cache(replay.trace_peak_tokens(steps, 16) // 16, 16, 3), steps)
+        first = first or _stacked(got)
+        assert float(np.quantile(_errors(got, first), 0.9)) < BF16_BETWEEN_SCHEDULES
+
+
 MATRIX_CORES = {
     # three heads on one key/value head (a wavefront's 16 rows are 5 tokens and a third), key entries of 48 (a slab and a
     # half), values of 80, a window that ends inside blocks of keys; the left side with five heads on one

@@ -75,6 +75,58 @@ ALIGNED = config([parallel(heads=4, kv_heads=2, dim=32, vdim=48, scale=0.1, coef
                  width=64, vocab=128)
 
 
+def random_config(seed: int) -> dict:
+    """A configuration drawn at random: two to six layers of both kinds in any order, head counts, sizes, windows and
+    constants of many kinds (sizes the matrix kernels take and sizes they refuse), readers of earlier layers' keys,
+    feed-forwards of every kind or none."""
+    import random
+    rng = random.Random(seed)
+
+    def mlp():
+        kind = rng.choice(["dense", "moe", "moe", None])
+        if kind is None:
+            return None
+        if kind == "dense":
+            return {"kind": "dense", "ff": rng.choice([40, 64, 100, 144])}
+        experts = rng.choice([2, 3, 6, 10, 16])
+        return feed_forward("moe", ff=rng.choice([16, 24, 48, 80]), experts=experts, top=rng.randint(1, min(experts, 4)),
+                            shared=rng.choice([0, 32, 72]))
+
+    layers, writers = [], []
+    for i in range(rng.randint(2, 6)):
+        if rng.random() < 0.6:
+            if writers and rng.random() < 0.4:
+                j = rng.choice(writers)
+                m = dict(layers[j]["mixer"], kv_from=j, heads=layers[j]["mixer"]["kv_heads"] * rng.choice([1, 2, 3, 5]),
+                         scale=rng.choice([0.1, 0.15, 0.22]))
+                m.pop("mask", None)
+                if rng.random() < 0.7:
+                    m["mask"] = {"size": rng.randint(1, 180)}
+            else:
+                kv, dim = rng.choice([1, 2, 3, 4]), rng.choice([16, 24, 32, 40, 48, 64, 80, 96, 128])
+                m = {"heads": kv * rng.choice([1, 2, 3, 4, 8]), "kv_heads": kv, "dim": dim, "vdim": rng.choice([16, 20, 32, 48, 64, 72, 96, 128]),
+                     "scale": rng.choice([0.1, 0.15, 0.22, dim ** -0.5])}
+                if rng.random() < 0.85:
+                    m["rot"] = {"base": rng.choice([5000.0, 80000.0, 2e6]), "dims": rng.choice([dim, dim // 4 * 2, 8])}
+                    if rng.random() < 0.7:
+                        m["rot"]["scaling"] = {"factor": rng.choice([1.5, 4.0, 20.0])}
+                if rng.random() < 0.85:
+                    m["mask"] = {"size": rng.choice([1, 7, 16, 33, 64, 100, 129, 150, 240])}
+                writers.append(i)
+            layers.append({"type": "attention", "mixer": m, "mlp": mlp()})
+        else:
+            kv = rng.choice([1, 2, 4])
+            layers.append(parallel(heads=kv * rng.choice([1, 2, 3, 4]), kv_heads=kv, dim=rng.choice([16, 32, 40, 64, 96, 128]),
+                                   vdim=rng.choice([16, 24, 32, 64, 128]), scale=rng.choice([0.08, 0.11, 0.2]),
+                                   coef=rng.choice([0.1, 0.3, 1.0]), every=rng.choice([0, 1, 16, 50, 100, 256]),
+                                   r_heads=rng.choice([1, 2, 3, 5, 8]), r_dim=rng.choice([8, 16, 24, 40, 64, 100, 128]),
+                                   r_vdim=rng.choice([8, 16, 32, 40, 64, 128]), tau=rng.choice([1.0, 4.0, 10.0, 50.0]),
+                                   rank=rng.choice([3, 8, 16, 32]), left_scale=rng.choice([0.5, 0.9, 1.0]),
+                                   right_scale=rng.choice([0.5, 1.0, 1.4]), mlp=mlp()))
+    return config(layers, width=rng.choice([64, 96, 136, 160, 192, 320]), vocab=rng.choice([100, 257, 384]),
+                  eps=rng.choice([1e-6, 1e-5]), logit_scale=rng.choice([0.3, 0.5, 1.0]), embedding_scale=rng.choice([1.0, 3.0, 8.0]))
+
+
 def make_weights(cfg: dict, seed: int, dtype=torch.bfloat16) -> dict:
     """name -> tensor for every tensor of the configuration's model (names and shapes as the engine's model tree
     lists them; the values are the tests' own)."""
@@ -94,7 +146,8 @@ def make_weights(cfg: dict, seed: int, dtype=torch.bfloat16) -> dict:
         elif name == "embed":
             t = torch.randn(shape, generator=g) * 0.5
         elif leaf == "router":
-            t = torch.randn(shape, generator=g) * 2.5 / shape[-1] ** 0.5
+            # (logits of order one whatever the embedding's multiplier: sigmoids that do not run into 0 or 1)
+            t = torch.randn(shape, generator=g) * 2.5 / shape[-1] ** 0.5 / min(4.0, float(cfg.get("embedding", {}).get("scale", 1.0)))
         else:
             t = torch.randn(shape, generator=g) * 1.3 / shape[-1] ** 0.5
         out[name] = t.to(dtype)
