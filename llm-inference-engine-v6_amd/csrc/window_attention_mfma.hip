@@ -6,7 +6,9 @@
 // its own position and so its own visible keys. Keys are walked in blocks of 32: the blocks that hold the first
 // keep_first tokens where they lie in front of the window, then the blocks from the window's start of the tile's
 // first row to the position of its last. The blocks of a tile are cut into `nsplit` runs (grid z); every run leaves
-// its maximum, sum and unscaled weighted values, which window_attention_finish joins in the order of the runs.
+// its maximum, sum and unscaled weighted values, which window_attention_finish joins in the order of the runs; where
+// there is one run (prompts) and a head has one map, the kernel can finish its rows itself (sink, a gate per head, a
+// scale) and write them in bfloat16.
 //
 //   S^T[key, row] = sum_d K[key, d] Q[row, d]     first operand: a key's entries as they lie in its page, 16 bytes a lane
 //   O^T[c, row]  += sum_key V^T[c, key] P^T[key, row]
@@ -39,7 +41,52 @@ struct WindowArgs {
     int max_blocks, T, nq, nk, nv, maps, per_value_head, dk, dv, page, page_shift, window, keep_first, nsplit;
     float scale, softcap;
     const float* slopes;        // [nq / maps] or null: a score loses slope (position - key)
+    // Where the keys are in one run and a head has one map, the kernel may finish a row itself instead of leaving its
+    // parts: out [T, ld_out] bfloat16 = acc / sum (the sum also holding e^(sink) where sinks [nq] are given), times
+    // out_scale and, where head_gate [T, ld_gate] is given, times sigmoid(head_gate[t, head]). out null: the parts.
+    bf16* out;
+    const float* sinks;
+    const float* head_gate;
+    int ld_out, ld_gate;
+    float out_scale;
 };
+
+// The end of a tile's walk: the row's parts into part_o / part_ml, or (a.out given) the finished row. l is the row's
+// whole sum already.
+template <int NVM>
+__device__ __forceinline__ void window_store(const WindowArgs& a, const f32x4 (&acc)[NVM], float m, float l, int nvt, int t, int qh,
+                                             int qd) {
+    if (a.out != nullptr) {
+        float f = 1.f, sum = l;
+        if (a.sinks != nullptr) {               // the sink joins like a run that holds one weight and no value
+            const float sk = a.sinks[qh];
+            const float top = fmaxf(m, sk);
+            f = m == -INFINITY ? 0.f : expf(m - top);
+            sum = fmaf(l, f, expf(sk - top));
+        }
+        float mul = a.out_scale * f / sum;
+        if (a.head_gate != nullptr) mul *= 1.0f / (1.0f + expf(-a.head_gate[static_cast<size_t>(t) * a.ld_gate + qh]));
+        bf16* orow = a.out + static_cast<size_t>(t) * a.ld_out + qh * a.dv + qd * 4;
+#pragma unroll
+        for (int c = 0; c < NVM; ++c) {
+            if (c < nvt) {
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = static_cast<__bf16>(acc[c][e] * mul);
+                *reinterpret_cast<bf16x4*>(orow + c * 16) = o;
+            }
+        }
+        return;
+    }
+    const size_t at = (static_cast<size_t>(blockIdx.z) * a.T + t) * a.nq + qh;
+    if (qd == 0) {
+        a.part_ml[at * 2] = m;
+        a.part_ml[at * 2 + 1] = l;
+    }
+#pragma unroll
+    for (int c = 0; c < NVM; ++c)
+        if (c < nvt) *reinterpret_cast<f32x4*>(a.part_o + at * a.dv + c * 16 + qd * 4) = acc[c];
+}
 
 // What is done to a raw score besides the scale: nothing, a cap, or a bias that grows with the distance.
 enum ScoreMode : int { kScorePlain = 0, kScoreCapped = 1, kScoreDistance = 2 };
@@ -228,14 +275,7 @@ __global__ __launch_bounds__(256, (DSM <= 2 && NVM <= 4) ? 4 : NVM <= 4 ? 3 : 2)
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (!valid) return;
-    const size_t at = (static_cast<size_t>(blockIdx.z) * a.T + t) * a.nq + qh;
-    if (qd == 0) {
-        a.part_ml[at * 2] = m;
-        a.part_ml[at * 2 + 1] = l;
-    }
-#pragma unroll
-    for (int c = 0; c < NVM; ++c)
-        if (c < nvt) *reinterpret_cast<f32x4*>(a.part_o + at * a.dv + c * 16 + qd * 4) = acc[c];
+    window_store<NVM>(a, acc, m, l, nvt, t, qh, qd);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -462,14 +502,7 @@ __global__ __launch_bounds__(256, 4) void window_attention_mfma_shared_kernel(Wi
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (!valid) return;
-    const size_t at = (static_cast<size_t>(blockIdx.z) * a.T + t) * a.nq + qh;
-    if (qd == 0) {
-        a.part_ml[at * 2] = m;
-        a.part_ml[at * 2 + 1] = l;
-    }
-#pragma unroll
-    for (int c = 0; c < NVM; ++c)
-        if (c < nvt) *reinterpret_cast<f32x4*>(a.part_o + at * a.dv + c * 16 + qd * 4) = acc[c];
+    window_store<NVM>(a, acc, m, l, nvt, t, qh, qd);
 }
 
 }  // namespace llme
@@ -483,13 +516,22 @@ extern "C" int llme_window_attention_mfma(const void* q, const void* k_cache, co
                                           const int* positions, const int* q_start, const int* block_table, int max_blocks, int T,
                                           int S, int max_new, int nq, int nk, int nv, int dk, int dv, int page, float scale,
                                           float softcap, int window, int keep_first, int nsplit, int staged, const float* slopes,
-                                          hipStream_t stream) {
+                                          void* out, int ld_out, const float* sinks, const float* head_gate, int ld_gate,
+                                          float out_scale, hipStream_t stream) {
     if (T <= 0 || S <= 0) return 0;
     if (nv <= 0 || nk % nv != 0 || nq % nk != 0 || max_new <= 0 || nsplit <= 0 || window < 0 || keep_first < 0) return kErrBadArgument;
     if (dk % 8 != 0 || dk > 128 || dv % 16 != 0 || dv > 128 || page % 16 != 0 || (page & (page - 1)) != 0) return kErrUnsupported;
     if (softcap > 0.f && slopes != nullptr) return kErrUnsupported;         // (capped and biased scores: the plain kernel)
+    // (finished rows: one run of keys, one map a head, rows of whole 8-byte pieces)
+    if (out != nullptr && (nsplit != 1 || nk != nv || ld_out % 4 != 0 || reinterpret_cast<uintptr_t>(out) % 8 != 0)) return kErrBadArgument;
     WindowArgs a;
     a.slopes = slopes;
+    a.out = static_cast<bf16*>(out);
+    a.ld_out = ld_out;
+    a.sinks = sinks;
+    a.head_gate = head_gate;
+    a.ld_gate = ld_gate;
+    a.out_scale = out_scale;
     a.q = static_cast<const bf16*>(q);
     a.k_cache = static_cast<const bf16*>(k_cache);
     a.v_cache = static_cast<const bf16*>(v_cache);

@@ -87,7 +87,8 @@ def qk_prepare(p: torch.Tensor, step, block_table: torch.Tensor | None, q_out: t
 
 
 declare("llme_window_attention_mfma", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
-                                       _i, _i, _vp, _vp])
+                                       _i, _i, _vp, _vp, _i, _vp, _vp, _i, _f, _vp])
+WINDOW_MFMA_FINISHES = True         # a step whose keys are in one run has its rows finished by the attention kernel (False: tests)
 WINDOW_MFMA_STAGED = True           # prompts' blocks of keys staged once a workgroup through LDS (False: measurements, tests)
 WINDOW_MFMA_MAX_ENTRIES = 128       # entries of a key or value head that the matrix-core kernel holds
 WINDOW_MFMA_MAX_RUNS = 32
@@ -125,7 +126,7 @@ def window_runs(step, rows_per_token: int, key_heads: int, window: int, keep_fir
     return max_new, runs
 
 
-def _fast_window_attention(q, k_cache, v_cache, step, block_table, nq, scale, softcap, window, keep_first, slopes=None):
+def _fast_window_attention(q, k_cache, v_cache, step, block_table, nq, scale, softcap, window, keep_first, slopes=None, finish=None):
     from .choices import choices_of
     if not window_mfma_fits(k_cache, v_cache, choices_of(step)) or (softcap > 0 and slopes is not None):
         return None
@@ -133,21 +134,43 @@ def _fast_window_attention(q, k_cache, v_cache, step, block_table, nq, scale, so
     _, nk, page, dk = k_cache.shape
     nv, dv = v_cache.shape[1], v_cache.shape[2]
     max_new, runs = window_runs(step, nq // nk, nk, window, keep_first)
-    part_o = step.buffer("window_attention.part_o", (runs, T, nq, dv), torch.float32)
-    part_ml = step.buffer("window_attention.part_ml", (runs, T, nq, 2), torch.float32)
+    out = gate = sinks = None
+    ld_out = ld_gate = 0
+    out_scale = 1.0
+    if finish is not None and runs == 1 and nk == nv and finish["mode"] in ("plain", "head_gate") and WINDOW_MFMA_FINISHES:
+        o = finish["out"]
+        if (o.dtype == torch.bfloat16 and o.stride(1) == 1 and o.stride(0) % 4 == 0 and o.data_ptr() % 8 == 0
+                and tuple(o.shape) == (T, nq * dv)):
+            # one run of keys: the kernel finishes its rows itself (the sink, the head's gate, the scale)
+            out, ld_out, out_scale, sinks = o, o.stride(0), float(finish.get("out_scale", 1.0)), finish.get("sinks")
+            if sinks is not None:
+                require(sinks, "sinks", torch.float32, (nq,))
+            if finish["mode"] == "head_gate":
+                gate = finish["gate"]
+                ld_gate = _columns(gate, "gate")
+                if tuple(gate.shape) != (T, nq):
+                    raise KernelError(f"window attention: gate must be [T, {nq}]")
+    if out is None:
+        part_o = step.buffer("window_attention.part_o", (runs, T, nq, dv), torch.float32)
+        part_ml = step.buffer("window_attention.part_ml", (runs, T, nq, 2), torch.float32)
+    else:
+        part_o = part_ml = None
     check(entry("llme_window_attention_mfma")(ptr(q), ptr(k_cache), ptr(v_cache), ptr(part_o), ptr(part_ml), ptr(step.positions),
                                               ptr(step.q_start), ptr(block_table), block_table.shape[1], T, step.num_seqs, max_new,
                                               nq, nk, nv, dk, dv, page, float(scale), float(softcap), int(window), int(keep_first),
-                                              runs, 1 if WINDOW_MFMA_STAGED else 0, ptr(slopes), stream()),
+                                              runs, 1 if WINDOW_MFMA_STAGED else 0, ptr(slopes), ptr(out), ld_out, ptr(sinks),
+                                              ptr(gate), ld_gate, out_scale, stream()),
           "window_attention_mfma")
-    return part_o, part_ml
+    return (part_o, part_ml) if out is None else "finished"
 
 
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, step, block_table: torch.Tensor, nq: int,
                      scale: float, softcap: float = 0.0, window: int = 0, keep_first: int = 0,
-                     slopes: torch.Tensor | None = None):
+                     slopes: torch.Tensor | None = None, finish: dict | None = None):
     """Every (token, query head) of the step over the keys of its request that it may see; slopes [heads] (32-bit): the
-    score of head h loses slopes[h] times the distance between query and key. Returns (part_o
+    score of head h loses slopes[h] times the distance between query and key. finish: what `window_attention_finish`
+    would be asked to do with the parts (out, mode, gate, sinks, out_scale); where the matrix-core kernel walks a
+    row's keys in one run it does that itself and "finished" is returned instead of the parts. Returns (part_o
     [runs, T, nq, dv], part_ml [runs, T, nq, 2]): per run of keys the unscaled weighted values, the maximum and the
     sum, which `window_attention_finish` joins."""
     T = q.shape[0]
@@ -164,7 +187,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     if slopes is not None:
         require(slopes, "slopes", torch.float32, (nq // (nk // nv),))
     if _fast_window_attention is not None:
-        parts = _fast_window_attention(q, k_cache, v_cache, step, block_table, nq, scale, softcap, window, keep_first, slopes)
+        parts = _fast_window_attention(q, k_cache, v_cache, step, block_table, nq, scale, softcap, window, keep_first, slopes, finish)
         if parts is not None:
             return parts
     part_o = step.buffer("window_attention.part_o", (1, T, nq, dv), torch.float32)

@@ -191,19 +191,20 @@ class WindowAttention(ProjectedMixer):
         else:
             ops.window.qk_prepare(p, step, None, q, None, None, nq, 0, None, self.inv_freq, self.rot_dims, self.wq, None,
                                   self.eps, self.rot_pairs, self.q_temp, dk=dim)
-        part_o, part_ml = ops.window.window_attention(q, k_cache, v_cache, step, table, nq, self.scale, self.softcap,
-                                                      self.window, self.keep_first, self.slopes)
+        # what is done with the runs' parts; where the keys are in one run the attention kernel may do it itself
         if M == 2:
-            ops.window.window_attention_finish(part_o, part_ml, o, n, "difference", lam=self.lam, eps=self.eps,
-                                               out_scale=(1.0 - self.diff) * scale)
+            finish = dict(out=o, mode="difference", lam=self.lam, eps=self.eps, out_scale=(1.0 - self.diff) * scale)
         elif self.gate == "heads":
-            ops.window.window_attention_finish(part_o, part_ml, o, n, "head_gate", gate=p[:, g_col:g_col + n], out_scale=scale,
-                                               sinks=self.sinks)
+            finish = dict(out=o, mode="head_gate", gate=p[:, g_col:g_col + n], out_scale=scale, sinks=self.sinks)
         elif self.gate:
-            ops.window.window_attention_finish(part_o, part_ml, o, n, "gate", gate=p[:, g_col:g_col + n * vdim], out_scale=scale,
-                                               sinks=self.sinks)
+            finish = dict(out=o, mode="gate", gate=p[:, g_col:g_col + n * vdim], out_scale=scale, sinks=self.sinks)
         else:
-            ops.window.window_attention_finish(part_o, part_ml, o, n, "plain", out_scale=scale, sinks=self.sinks)
+            finish = dict(out=o, mode="plain", out_scale=scale, sinks=self.sinks)
+        parts = ops.window.window_attention(q, k_cache, v_cache, step, table, nq, self.scale, self.softcap, self.window,
+                                            self.keep_first, self.slopes, finish=finish)
+        if parts != "finished":
+            out = finish.pop("out")
+            ops.window.window_attention_finish(parts[0], parts[1], out, n, **finish)
 
 
 register_part("mixer", "window_attention", WindowAttention)

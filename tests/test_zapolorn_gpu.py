@@ -206,6 +206,31 @@ def test_the_matrix_core_attention_at_other_sizes(tmp_path, name):
         assert _mean(got, ref) < 6e-2
 
 
+@pytest.mark.parametrize("name", ["three_heads", "many_heads"])
+def test_rows_finished_by_the_attention_kernel_are_what_the_finishing_kernel_makes(tmp_path, name):
+    """Where a step's keys are walked in one run (prompts) the matrix-core kernel applies the sink, the head's gate and the
+    side's scale itself and writes the rows; the same steps through the parts and the finishing kernel give the same rows
+    up to the rounding of the stored values."""
+    from llmengine.ops import window
+    cfg = MATRIX_CORES[name]
+    engine, weights = _engine(tmp_path, cfg, 23, "bf16")
+    V = cfg["vocab"]
+    requests = {"a": _tokens(333, V, 5), "b": _tokens(70, V, 6), "c": _tokens(17, V, 7)}
+    for steps in (replay.whole(requests), replay.portions(requests, sizes=(65, 16, 130, 23))):
+        got = {}
+        for fused in (True, False):
+            window.WINDOW_MFMA_FINISHES = fused
+            try:
+                got[fused] = _stacked(replay.run_trace(engine, engine.new_cache(replay.trace_peak_tokens(steps, 16) // 16, 16, 3), steps))
+            finally:
+                window.WINDOW_MFMA_FINISHES = True
+        assert _mean(replay_rows(got[True]), got[False]) < 3e-3 and _worst(replay_rows(got[True]), got[False]) < 3e-2
+
+
+def replay_rows(stacked: dict) -> dict:
+    return {rid: {p: rows[p] for p in range(len(rows))} for rid, rows in stacked.items()}
+
+
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 def test_a_batch_of_unequal_requests_against_each_alone(tmp_path, dtype):
     cfg = zm.ALIGNED
